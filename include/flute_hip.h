@@ -1,0 +1,194 @@
+/*
+ * flute_hip.h — C ABI of the MI355X (gfx950) idxN LUT-palettized linear layer.
+ *
+ * One shared library, libflute_hip.so, plain pointers and sizes, no framework
+ * types.  Every pointer named "device" must be memory of the current HIP
+ * device; `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ * Launches are asynchronous: no entry point synchronises or copies to the host.
+ *
+ * Each entry point names the upstream interface it replaces (paths relative to
+ * the upstream tree's src/flute_extended/).  Upstream exposes these through
+ * pybind11 with torch::Tensor arguments (src/bindings.cpp:230-546); here the
+ * same operands arrive as raw pointers plus the sizes upstream derives from
+ * the tensors.
+ *
+ * Error model: every function returns FLUTE_OK or one of the FLUTE_ERR_* codes;
+ * the message of the last failure on the calling thread is available from
+ * flute_last_error().  All argument validation happens before the device is
+ * touched, so the refusal paths can be exercised on a machine without a GPU.
+ * There is no fallback of any kind: a shape or dtype the kernels do not serve
+ * is refused with FLUTE_ERR_UNSUPPORTED.
+ */
+#ifndef FLUTE_HIP_H
+#define FLUTE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum flute_status {
+    FLUTE_OK = 0,
+    FLUTE_ERR_INVALID = 1,      /* contract violation (shape, size, alignment, NULL) */
+    FLUTE_ERR_UNSUPPORTED = 2,  /* valid but outside what the kernels serve          */
+    FLUTE_ERR_HIP = 3,          /* a HIP runtime call failed                          */
+    FLUTE_ERR_NOMEM = 4         /* workspace allocation failed                        */
+} flute_status;
+
+typedef enum flute_dtype {
+    FLUTE_F16 = 0,
+    FLUTE_BF16 = 1,
+    FLUTE_F32 = 2
+} flute_dtype;
+
+/*
+ * One palettized weight, as the upstream kernel entries receive it
+ * (src/kernel_gemv.cu:322-333, src/kernel_gemv_splitk.cu:813-830):
+ *
+ *   W[n, k] = lut1[n / group_size][idx1[n, k]]  (+ the same for stream 2)
+ *   y       = x W^T + (x resB^T) resA^T + bias
+ *
+ * q1/q2   idxN blobs (flute_extended/idxN.py:37-55), N*K*b/8 bytes, 16-byte aligned
+ * lut1/2  [ceil(N/group_size), 2^b] in lut_dtype, contiguous
+ * b2 == 0 means "single stream" and q2/lut2 are ignored
+ * resB    (R, K), resA (N, R), bias (N,) in the ACTIVATION dtype, or NULL / R = 0
+ * signs   (K,) fp32 +-1: when non-NULL the input is rotated first, x <- x @ T
+ *         (fht.py:19-35); awq (K,) fp32 then selects ((x*s) @ T) / s
+ */
+typedef struct flute_linear {
+    const void *q1;
+    const void *lut1;
+    const void *q2;
+    const void *lut2;
+    const void *resB;
+    const void *resA;
+    const void *bias;
+    const float *signs;
+    const float *awq;
+    int64_t q1_bytes;
+    int64_t q2_bytes;
+    int32_t lut_rows;      /* rows of lut1 (and of lut2): must equal ceil(N/group_size) */
+    int32_t N;
+    int32_t K;
+    int32_t R;
+    int32_t b1;
+    int32_t b2;
+    int32_t group_size;
+    int32_t lut_dtype;     /* FLUTE_F16 or FLUTE_BF16 */
+    int32_t rot_block;     /* 0: rotation over the descending power-of-two segments of K
+                              (upstream's transform); > 0: equal blocks of this many
+                              columns, each normalised by 1/sqrt(rot_block) */
+} flute_linear;
+
+/* Library identity and diagnostics. */
+int flute_abi_version(void);
+const char *flute_last_error(void);
+/* Name of the code-object architecture the kernels were built for ("gfx950"). */
+const char *flute_target_arch(void);
+
+/*
+ * M = 1 LUT GEMV:  y[1, N] = linear(x[1, K]).
+ * Replaces qgemm_gemv_stream, qgemm_gemv_fht_stream, qgemm_gemv_splitk_stream
+ * and qgemm_gemv_splitk_fht_stream (src/bindings.cpp:277-354): rotation is
+ * selected by w->signs, the K split by `split` (0 = library policy,
+ * flute_pick_split; otherwise 1 <= split, split must divide K/64).
+ * x and y are act_dtype (FLUTE_F16 or FLUTE_BF16).  Deterministic: partial
+ * sums are folded in a fixed order, so repeated calls are bit identical.
+ */
+flute_status flute_gemv(const flute_linear *w, const void *x, void *y,
+                        int act_dtype, int split, void *stream);
+
+/*
+ * Merged gate+up GEMV with the SiLU*mul epilogue, M = 1:
+ *   h[n] = silu(gate(x)[n]) * up(x)[n],   silu(v) = v / (1 + exp(-v)), fp32,
+ * one rounding to act_dtype.  Replaces qgemm_gemv_mlp (src/bindings.cpp:378-384,
+ * src/kernel_gemv_mlp.cu:536-691).  gate and up must agree in N and K; all
+ * other fields may differ.
+ */
+flute_status flute_gemv_mlp(const flute_linear *gate, const flute_linear *up,
+                            const void *x, void *h, int act_dtype, int split,
+                            void *stream);
+
+/*
+ * Several weights sharing one input row, one launch (the QKV merge):
+ * outs[i][1, N_i] = linear_i(x).  Replaces qgemm_gemv_multi
+ * (src/bindings.cpp:368-373, src/kernel_gemv_multi.cu).  1 <= count <= 4, all K
+ * equal.
+ */
+flute_status flute_gemv_multi(const flute_linear *segs, int count, const void *x,
+                              void *const *outs, int act_dtype, int split,
+                              void *stream);
+
+/*
+ * The whole decode MLP block for one token, two dependent launches on `stream`
+ * (merged gate+up with SiLU*mul, then down):  y = down( silu(gate(x)) * up(x) ).  h is caller-provided scratch
+ * of gate->N elements in act_dtype.  Mirrors FusedPalettizedMLP.forward at
+ * M = 1 (scripts/palettized_modules.py:1673-1682).
+ */
+flute_status flute_mlp_block(const flute_linear *gate, const flute_linear *up,
+                             const flute_linear *down, const void *x, void *h,
+                             void *y, int act_dtype, void *stream);
+
+/*
+ * Small-M / prefill LUT GEMM:  C[M, N] = A[M, K] @ W^T (+ stream 2, residual,
+ * bias), fp32 accumulate on MFMA, one rounding to act_dtype.  Replaces
+ * qgemm_per_group_lut / qgemm_cutlass_streaming (src/bindings.cpp:231-251,
+ * src/kernel_streaming.cu:2297-2443) and qgemm_dual_stream
+ * (src/bindings.cpp:257-270).  The MFMA operand type follows lut_dtype, so the
+ * dequantised tile is exactly the LUT entry; A is converted to that type if it
+ * differs.  lda = row stride of A in elements (>= K), ldc likewise for C.
+ */
+flute_status flute_gemm(const flute_linear *w, const void *A, void *C, int M,
+                        int64_t lda, int64_t ldc, int act_dtype, void *stream);
+
+/*
+ * Dequantise one stream to a dense row-major [N, K] matrix in lut_dtype,
+ * through the same tile decoder the GEMM uses.  which = 1 or 2.  Serves the
+ * bit-exact tile check that upstream runs against dequantize_reference
+ * (test_flute.py:172-223) and the role of its scalar differential twin
+ * (src/kernel_debug_simple.cu).
+ */
+flute_status flute_dequant(const flute_linear *w, int which, void *W_out,
+                           void *stream);
+
+/*
+ * Walsh-Hadamard rotation of M rows of length K (fht.py:19-35):
+ *   adjoint == 0:  out = x @ T      = ((x @ H) * s) / sqrt(b) per segment
+ *   adjoint != 0:  out = x @ T^T    = ((x * s) @ H) / sqrt(b) per segment
+ *   awq != NULL (forward only): out = ((x * awq) @ T) / awq, fp32, true division
+ * Segments are the descending powers of two of K when block == 0, or equal
+ * blocks of `block` columns (a power of two dividing K) otherwise.  out == x is
+ * allowed.  dtype is FLUTE_F16, FLUTE_BF16 or FLUTE_F32 for both x and out.
+ * Replaces fht_forward, fht_backward, fht_inplace_ and fht_forward_awq
+ * (src/bindings.cpp:386-399, src/kernel_fht.cu:335-397).
+ * Contract: K % 32 == 0, 32 <= K <= 65504, every segment <= 16384
+ * (fht.py:381-390).
+ */
+flute_status flute_fht(const void *x, const float *signs, const float *awq,
+                       void *out, int M, int K, int dtype, int adjoint, int block,
+                       void *stream);
+
+/*
+ * The K-split the library would choose for an (N, K) GEMV on this device
+ * (the MI355X restatement of gemv_pick_split, src/gemv_host.cpp:29-38).
+ * Pure host arithmetic: usable without a GPU.
+ */
+int flute_pick_split(int N, int K);
+
+/* LDS bytes one GEMV workgroup needs for this weight (0 when the weight is
+ * refused); the host-side gates mirror it (flute_extended/__init__.py:643-665). */
+int64_t flute_gemv_lds_bytes(const flute_linear *w, int split);
+
+/* Validate a weight descriptor exactly as the launchers do, without touching
+ * the device.  mode: 0 = GEMV, 1 = GEMM. */
+flute_status flute_validate(const flute_linear *w, int mode);
+
+/* Release the per-device split-K workspaces (also done at process exit). */
+void flute_release_workspaces(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLUTE_HIP_H */

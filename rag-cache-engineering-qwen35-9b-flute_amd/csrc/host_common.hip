@@ -1,0 +1,177 @@
+// Validation, split policy, workspace and the small identity entry points.
+#include "host_common.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+namespace flute {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+static bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+flute_status validate_linear(const flute_linear *w, int mode, const char *who) {
+    FLUTE_REQUIRE(w != nullptr, FLUTE_ERR_INVALID, "%s: weight descriptor is NULL", who);
+    FLUTE_REQUIRE(w->b1 >= 1 && w->b1 <= 4, FLUTE_ERR_INVALID,
+                  "%s: bitwidth must be 1, 2, 3 or 4 (got %d)", who, w->b1);
+    FLUTE_REQUIRE(w->b2 >= 0 && w->b2 <= 4, FLUTE_ERR_INVALID,
+                  "%s: bitwidth2 must be 0 (single stream) or 1..4 (got %d)", who, w->b2);
+    FLUTE_REQUIRE(w->K > 0 && w->K % 64 == 0, FLUTE_ERR_INVALID,
+                  "%s: K must be a positive multiple of 64, the idxN blob's 64-k tiles (got K=%d)",
+                  who, w->K);
+    FLUTE_REQUIRE(w->N > 0 && w->N % 128 == 0, FLUTE_ERR_INVALID,
+                  "%s: the idxN layout requires N %% 128 == 0 (got N=%d)", who, w->N);
+    const int gs = w->group_size;
+    FLUTE_REQUIRE(is_pow2(gs) && gs >= 16 && gs <= 2048, FLUTE_ERR_INVALID,
+                  "%s: group_size must be one of 16/32/64/128/256/512/1024/2048 (got %d)", who, gs);
+    FLUTE_REQUIRE(w->lut_dtype == FLUTE_F16 || w->lut_dtype == FLUTE_BF16, FLUTE_ERR_INVALID,
+                  "%s: lut dtype must be float16 or bfloat16", who);
+    FLUTE_REQUIRE(w->q1 != nullptr && w->lut1 != nullptr, FLUTE_ERR_INVALID,
+                  "%s: stream-1 indices/lut must not be NULL", who);
+    const int64_t want1 = (int64_t)w->N * w->K * w->b1 / 8;
+    FLUTE_REQUIRE(w->q1_bytes == want1, FLUTE_ERR_INVALID,
+                  "%s: stream-1 byte count %lld is not N*K*%d/8 = %lld (N=%d, K=%d)", who,
+                  (long long)w->q1_bytes, w->b1, (long long)want1, w->N, w->K);
+    FLUTE_REQUIRE(aligned(w->q1, 16), FLUTE_ERR_INVALID,
+                  "%s: stream-1 indices must be 16-byte aligned", who);
+    FLUTE_REQUIRE(aligned(w->lut1, 2), FLUTE_ERR_INVALID, "%s: lut misaligned", who);
+    const int rows = (w->N + gs - 1) / gs;
+    FLUTE_REQUIRE(w->lut_rows == rows, FLUTE_ERR_INVALID,
+                  "%s: lut must be [ceil(N/group_size), 2^bitwidth] = [%d, %d] (got %d rows)", who,
+                  rows, 1 << w->b1, w->lut_rows);
+    if (w->b2 > 0) {
+        FLUTE_REQUIRE(w->q2 != nullptr && w->lut2 != nullptr, FLUTE_ERR_INVALID,
+                      "%s: a second stream needs both indices2 and lut2", who);
+        const int64_t want2 = (int64_t)w->N * w->K * w->b2 / 8;
+        FLUTE_REQUIRE(w->q2_bytes == want2, FLUTE_ERR_INVALID,
+                      "%s: stream-2 byte count %lld != N*K*%d/8 = %lld", who,
+                      (long long)w->q2_bytes, w->b2, (long long)want2);
+        FLUTE_REQUIRE(aligned(w->q2, 16), FLUTE_ERR_INVALID,
+                      "%s: stream-2 indices must be 16-byte aligned", who);
+    }
+    FLUTE_REQUIRE((w->resA != nullptr) == (w->resB != nullptr), FLUTE_ERR_INVALID,
+                  "%s: resB and resA must be supplied together", who);
+    FLUTE_REQUIRE((w->resA != nullptr) == (w->R > 0), FLUTE_ERR_INVALID,
+                  "%s: residual rank %d does not match the residual pointers", who, w->R);
+    FLUTE_REQUIRE(w->R >= 0 && w->R <= 256, FLUTE_ERR_INVALID,
+                  "%s: residual rank must be 0..256 (got R=%d)", who, w->R);
+    FLUTE_REQUIRE(w->awq == nullptr || w->signs != nullptr, FLUTE_ERR_INVALID,
+                  "%s: awq scale only exists as a companion to the rotation signs", who);
+    if (w->signs != nullptr) {
+        FLUTE_REQUIRE(mode == 0, FLUTE_ERR_UNSUPPORTED,
+                      "%s: the fused rotation is a GEMV prologue; rotate the GEMM input with "
+                      "flute_fht first",
+                      who);
+        FLUTE_REQUIRE(w->K % 32 == 0 && w->K >= 32 && w->K <= 65504, FLUTE_ERR_INVALID,
+                      "%s: rotation needs K %% 32 == 0 and 32 <= K <= 65504 (got %d)", who, w->K);
+        const Segs sg = make_segments(w->K, 0);
+        FLUTE_REQUIRE(sg.len[0] <= 16384, FLUTE_ERR_UNSUPPORTED,
+                      "%s: rotation segment %d exceeds 16384 columns", who, sg.len[0]);
+    }
+    return FLUTE_OK;
+}
+
+// One workgroup holds a 64 KB table, so two fit a CU; three waves of 256
+// workgroups keep every CU busy while the tail of one wave drains.
+int pick_split_tiles(int tiles, int G) {
+    if (tiles <= 0 || G <= 0) return 1;
+    const int target = 3 * kNumCU;
+    int best = 1;
+    long best_cost = -1;
+    for (int d = 1; d <= G; ++d) {
+        if (G % d) continue;
+        if (G / d < 2 && d > 1) continue;          // keep two 64-k tiles per workgroup
+        const long wgs = (long)tiles * d;
+        const long cost = wgs > target ? (wgs - target) * 2 : (target - wgs);
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best = d;
+        }
+    }
+    return best;
+}
+
+struct Workspace {
+    float *P = nullptr;
+    int *tickets = nullptr;
+    size_t floats = 0;
+    size_t ints = 0;
+};
+
+static std::mutex g_ws_mu;
+static std::unordered_map<int, Workspace> g_ws;
+static std::vector<void *> g_retired;   // outgrown buffers, freed at release
+
+flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float **P,
+                           int **tickets) {
+    int dev = 0;
+    FLUTE_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> guard(g_ws_mu);
+    Workspace &ws = g_ws[dev];
+    if (ws.floats < floats) {
+        size_t want = ws.floats ? ws.floats : (size_t)1 << 20;
+        while (want < floats) want *= 2;
+        float *fresh = nullptr;
+        if (hipMalloc((void **)&fresh, want * sizeof(float)) != hipSuccess) {
+            set_error("split-K workspace: hipMalloc of %zu bytes failed", want * sizeof(float));
+            return FLUTE_ERR_NOMEM;
+        }
+        if (ws.P) g_retired.push_back(ws.P);       // kernels in flight may still read it
+        ws.P = fresh;
+        ws.floats = want;
+    }
+    if (ws.ints < ints) {
+        size_t want = ws.ints ? ws.ints : (size_t)1 << 14;
+        while (want < ints) want *= 2;
+        int *fresh = nullptr;
+        if (hipMalloc((void **)&fresh, want * sizeof(int)) != hipSuccess) {
+            set_error("split-K workspace: hipMalloc of %zu bytes failed", want * sizeof(int));
+            return FLUTE_ERR_NOMEM;
+        }
+        FLUTE_HIP_CHECK(hipMemsetAsync(fresh, 0, want * sizeof(int), stream));
+        if (ws.tickets) g_retired.push_back(ws.tickets);
+        ws.tickets = fresh;
+        ws.ints = want;
+    }
+    *P = ws.P;
+    *tickets = ws.tickets;
+    return FLUTE_OK;
+}
+
+}  // namespace flute
+
+extern "C" {
+
+int flute_abi_version(void) { return 1; }
+
+const char *flute_last_error(void) { return flute::g_error; }
+
+const char *flute_target_arch(void) { return "gfx950"; }
+
+flute_status flute_validate(const flute_linear *w, int mode) {
+    return flute::validate_linear(w, mode, "flute_validate");
+}
+
+void flute_release_workspaces(void) {
+    std::lock_guard<std::mutex> guard(flute::g_ws_mu);
+    for (auto &kv : flute::g_ws) {
+        if (kv.second.P) (void)hipFree(kv.second.P);
+        if (kv.second.tickets) (void)hipFree(kv.second.tickets);
+    }
+    flute::g_ws.clear();
+    for (void *p : flute::g_retired) (void)hipFree(p);
+    flute::g_retired.clear();
+}
+
+}  // extern "C"
