@@ -17,14 +17,6 @@ int env_int(const char *name, int fallback) {
     return std::atoi(e);
 }
 
-// log2 of the LDS bytes one workgroup may spend on lookup tables.
-int table_budget_log2() {
-    int v = env_int("FLUTE_GEMV_TABLE_LOG2", 16);
-    if (v < 12) v = 12;
-    if (v > 17) v = 17;
-    return v;
-}
-
 int entries_log2(int bits) { return bits == 3 ? 6 : 8; }
 int entry_bytes_log2(int bits) { return bits >= 3 ? 2 : (bits == 2 ? 3 : 4); }
 
@@ -32,16 +24,72 @@ struct Plan {
     GemvParams p;
     size_t lds_bytes;
     int grid_x;
+    int threads;
     int total_tickets;
-    size_t ws_floats;
+    size_t p_floats;        // partial sums
+    size_t xb_floats;       // residual coefficients
+    size_t xrot_halves;     // pre-rotated inputs of weights that carry a residual
     bool lut_bf16;
+    // pre-kernels: residual coefficients (and the rotation they need)
+    struct Pre {
+        const uint16_t *resB;
+        const float *signs, *awq;
+        int R, seg;
+        size_t xb_off, xrot_off;
+    } pre[kGemvMaxSegs];
+    int npre;
+    int rot_block;
 };
+
+// Shape of the launch for `rows` output rows over G tiles of K.  A workgroup
+// owns `rw` rows; without a K split nothing is exchanged between workgroups, so
+// the split stays 1 as long as the row slices alone give every CU at least two
+// workgroups.
+void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *waves) {
+    int best_rw = env_int("FLUTE_GEMV_RW", 0);
+    if (best_rw != 8 && best_rw != 16 && best_rw != 32) {
+        best_rw = 8;
+        for (int cand : {32, 16, 8}) {
+            if (rows / cand >= 2 * kNumCU + kNumCU / 2) { best_rw = cand; break; }
+        }
+    }
+    int sp = split_req;
+    if (sp > 0) {
+        // a wavefront load spans 32/rw tiles of K: widen the slices until the K
+        // range of one split is a whole number of loads
+        while (G % sp == 0 && (G / sp) % (32 / best_rw) != 0 && best_rw < 32) best_rw *= 2;
+    } else {
+        sp = 1;
+        const long slices = rows / best_rw;
+        const int gpi = 32 / best_rw;
+        if (slices < 2 * kNumCU) {
+            // narrow output: split K until the grid reaches about three workgroups per CU
+            long best_cost = -1;
+            for (int d = 1; d <= G; ++d) {
+                if (G % d || (G / d) % gpi) continue;
+                if (G / d < 4 * gpi && d > 1) continue;
+                const long wgs = slices * d;
+                const long target = 3 * kNumCU;
+                const long cost = wgs > target ? 2 * (wgs - target) : target - wgs;
+                if (best_cost < 0 || cost < best_cost) { best_cost = cost; sp = d; }
+            }
+        }
+        while ((G / sp) % (32 / best_rw) != 0 && best_rw < 32) best_rw *= 2;
+    }
+    *rw = best_rw;
+    *split = sp;
+    int wv = env_int("FLUTE_GEMV_WAVES", 0);
+    if (wv != 1 && wv != 2 && wv != 4 && wv != 8) {
+        const int units = (G / sp) / (32 / best_rw);
+        wv = units >= 16 ? 8 : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
+    }
+    *waves = wv;
+}
 
 // Fill a launch plan for `count` weights that share x.  silu_mul couples
 // weights 0 and 1 into one output.
 flute_status make_plan(const flute_linear *segs, int count, const void *x, void *const *outs,
-                       int act_dtype, int split, int silu_mul, int fht_block, const char *who,
-                       Plan *plan) {
+                       int act_dtype, int split, int silu_mul, const char *who, Plan *plan) {
     FLUTE_REQUIRE(count >= 1 && count <= kGemvMaxSegs, FLUTE_ERR_INVALID,
                   "%s: 1..%d weights per launch (got %d)", who, kGemvMaxSegs, count);
     FLUTE_REQUIRE(x != nullptr, FLUTE_ERR_INVALID, "%s: x is NULL", who);
@@ -56,6 +104,8 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
                       segs[0].K);
         FLUTE_REQUIRE(segs[i].lut_dtype == segs[0].lut_dtype, FLUTE_ERR_UNSUPPORTED,
                       "%s: all weights of one launch must share the LUT dtype", who);
+        FLUTE_REQUIRE(segs[i].rot_block == segs[0].rot_block, FLUTE_ERR_UNSUPPORTED,
+                      "%s: all weights of one launch must share the rotation block", who);
     }
     const bool lut_bf16 = segs[0].lut_dtype == FLUTE_BF16;
     FLUTE_REQUIRE(!(lut_bf16 && act_dtype == FLUTE_F16), FLUTE_ERR_UNSUPPORTED,
@@ -69,22 +119,88 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     }
     const int K = segs[0].K;
     const int G = K / 64;
+    FLUTE_REQUIRE(split <= 0 || G % split == 0, FLUTE_ERR_INVALID,
+                  "%s: split %d must divide K/64 = %d", who, split, G);
 
     GemvParams &p = plan->p;
     std::memset(&p, 0, sizeof(p));
-    int tiles = 0;
-    for (int i = 0; i < count; ++i)
-        tiles += (segs[i].N / 128) * (segs[i].b2 > 0 ? 2 : 1);
-    if (split <= 0) split = pick_split_tiles(tiles, G);
-    FLUTE_REQUIRE(split >= 1 && G % split == 0, FLUTE_ERR_INVALID,
-                  "%s: split %d must divide K/64 = %d", who, split, G);
+    int rows = 0;
+    for (int i = 0; i < (silu_mul ? 1 : count); ++i) rows += segs[i].N;
+    int rw, waves;
+    choose_shape(rows, G, split, &rw, &split, &waves);
+    FLUTE_REQUIRE((G / split) % (32 / rw) == 0, FLUTE_ERR_UNSUPPORTED,
+                  "%s: K/64/split = %d is not a whole number of wavefront loads", who, G / split);
     const int gs_tiles = G / split;
     const int kc = gs_tiles * 64;
+    const int spt = 128 / rw;
 
-    bool any_rot = false;
-    for (int i = 0; i < count; ++i) any_rot |= segs[i].signs != nullptr;
+    bool any_fused_rot = false;
+    const int fht_block = segs[0].rot_block;
+    plan->npre = 0;
+    plan->rot_block = fht_block;
+    size_t xb_off = 0, xrot_off = 0;
+    int n0 = 0, col = 0, ticket = 0;
+    size_t tab_bytes = 0;
+    // LDS: tables/scratch | x slice | row sums.  Two workgroups per CU when possible.
+    int budget = env_int("FLUTE_GEMV_TABLE_LOG2", 0);
+    if (budget < 12 || budget > 17) budget = (kc * 2 + 4096 + 65536 <= kLdsPerCU / 2) ? 16 : 15;
+    for (int i = 0; i < count; ++i) {
+        const flute_linear &w = segs[i];
+        GemvSeg &sg = p.seg[i];
+        sg.resA = (const uint16_t *)w.resA;
+        sg.bias = (const uint16_t *)w.bias;
+        sg.out = (uint16_t *)outs[i];
+        sg.N = w.N;
+        sg.R = w.R;
+        sg.gs = w.group_size;
+        sg.lut_rows = w.lut_rows;
+        sg.nstreams = w.b2 > 0 ? 2 : 1;
+        sg.n0 = n0;
+        sg.col0 = (silu_mul && i == 1) ? 0 : col;
+        sg.ticket0 = (silu_mul && i == 1) ? 0 : ticket;
+        n0 += w.N;
+        if (!(silu_mul && i == 1)) {
+            col += (w.N / 128) * spt;
+            ticket += (w.N / 128) * spt;
+        }
+        if (w.R > 0) {
+            // the residual needs x . resB[r] before any row can finish: computed by a
+            // small kernel in front, on the rotated input when the weight is rotated
+            Plan::Pre &pre = plan->pre[plan->npre++];
+            pre.resB = (const uint16_t *)w.resB;
+            pre.signs = w.signs;
+            pre.awq = w.awq;
+            pre.R = w.R;
+            pre.seg = i;
+            pre.xb_off = xb_off;
+            pre.xrot_off = xrot_off;
+            xb_off += (size_t)((w.R + 3) & ~3);
+            if (w.signs) xrot_off += (size_t)K;
+            sg.signs = nullptr;                     // the kernel reads the pre-rotated row
+            sg.awq = nullptr;
+        } else {
+            sg.signs = w.signs;
+            sg.awq = w.awq;
+            any_fused_rot |= w.signs != nullptr;
+        }
+        const int ngrp_log2 = w.group_size >= 128 ? 0 : ilog2(128 / w.group_size);
+        for (int st = 0; st < sg.nstreams; ++st) {
+            GemvStream &gs = sg.st[st];
+            gs.q = (const uint8_t *)(st ? w.q2 : w.q1);
+            gs.lut = (const uint16_t *)(st ? w.lut2 : w.lut1);
+            gs.bits = st ? w.b2 : w.b1;
+            int es = budget - entries_log2(gs.bits) - ngrp_log2;
+            if (es > 8) es = 8;
+            if (es < entry_bytes_log2(gs.bits)) es = entry_bytes_log2(gs.bits);
+            gs.es = es;
+            const size_t tb = ((size_t)1 << (entries_log2(gs.bits) + es)) << ngrp_log2;
+            if (tb > tab_bytes) tab_bytes = tb;
+        }
+    }
     size_t scratch = 0;
     if (fht_block > 0) {
+        bool any_rot = false;
+        for (int i = 0; i < count; ++i) any_rot |= segs[i].signs != nullptr;
         FLUTE_REQUIRE(any_rot, FLUTE_ERR_INVALID, "%s: a rotation block needs rotation signs", who);
         FLUTE_REQUIRE(is_pow2(fht_block) && fht_block >= 32 && fht_block <= 16384 &&
                           K % fht_block == 0,
@@ -94,67 +210,17 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
                       "%s: K slice %d of split %d is not a whole number of %d-column rotation "
                       "blocks",
                       who, kc, split, fht_block);
-        scratch = (size_t)kc * 4;
-    } else if (any_rot) {
+        if (any_fused_rot) scratch = (size_t)kc * 4;
+    } else if (any_fused_rot) {
         scratch = (size_t)make_segments(K, 0).len[0] * 4;
     }
     p.fht_block = fht_block;
-
-    const int budget = table_budget_log2();
-    size_t tab_bytes = 0;
-    int njobs = 0, col = 0, n0 = 0, r0 = 0, ticket = 0;
-    int ntot = 0;
-    for (int i = 0; i < count; ++i) ntot += segs[i].N;
-    for (int i = 0; i < count; ++i) {
-        const flute_linear &w = segs[i];
-        GemvSeg &sg = p.seg[i];
-        sg.resB = (const uint16_t *)w.resB;
-        sg.resA = (const uint16_t *)w.resA;
-        sg.bias = (const uint16_t *)w.bias;
-        sg.signs = w.signs;
-        sg.awq = w.awq;
-        sg.out = (uint16_t *)outs[i];
-        sg.N = w.N;
-        sg.R = w.R;
-        sg.gs = w.group_size;
-        sg.lut_rows = w.lut_rows;
-        const int nstreams = w.b2 > 0 ? 2 : 1;
-        sg.nslots = nstreams * split;
-        sg.arrivals = sg.nslots;
-        sg.n0 = n0;
-        sg.r0 = ntot + r0;
-        sg.ticket0 = (silu_mul && i == 1) ? p.seg[0].ticket0 : ticket;
-        n0 += w.N;
-        r0 += w.R;
-        if (!(silu_mul && i == 1)) ticket += w.N / 128;
-        const int ngrp_log2 = w.group_size >= 128 ? 0 : ilog2(128 / w.group_size);
-        for (int st = 0; st < nstreams; ++st) {
-            GemvJob &jb = p.job[njobs++];
-            jb.q = (const uint8_t *)(st ? w.q2 : w.q1);
-            jb.lut = (const uint16_t *)(st ? w.lut2 : w.lut1);
-            jb.bits = st ? w.b2 : w.b1;
-            jb.seg = i;
-            jb.tile0 = col;
-            jb.ntiles = w.N / 128;
-            jb.slot0 = st * split;
-            int es = budget - entries_log2(jb.bits) - ngrp_log2;
-            if (es > 8) es = 8;
-            if (es < entry_bytes_log2(jb.bits)) es = entry_bytes_log2(jb.bits);
-            jb.es = es;
-            const size_t tb = ((size_t)1 << (entries_log2(jb.bits) + es)) << ngrp_log2;
-            if (tb > tab_bytes) tab_bytes = tb;
-            col += jb.ntiles;
-        }
-    }
-    if (silu_mul) {
-        const int total = p.seg[0].nslots + p.seg[1].nslots;
-        p.seg[0].arrivals = p.seg[1].arrivals = total;
-    }
-    p.njobs = njobs;
+    p.nsegs = count;
     p.K = K;
     p.split = split;
     p.gs_tiles = gs_tiles;
-    p.p_stride = (ntot + r0 + 31) & ~31;
+    p.lpg_log2 = ilog2(2 * rw);
+    p.p_stride = (n0 + 31) & ~31;
     p.silu_mul = silu_mul;
     p.act_bf16 = act_dtype == FLUTE_BF16;
     p.x = (const uint16_t *)x;
@@ -163,45 +229,90 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     region0 = (region0 + 255) & ~(size_t)255;
     p.lds_x = (int)region0;
     p.lds_red = p.lds_x + ((kc * 2 + 15) & ~15);
-    p.lds_xb = p.lds_red + 128 * 4;
-    plan->lds_bytes = (size_t)p.lds_xb + kGemvMaxRank * 4 + 16;
+    plan->lds_bytes = (size_t)p.lds_red + 2 * 8 * 32 * 4 + 16;
     FLUTE_REQUIRE(plan->lds_bytes <= (size_t)kLdsPerCU, FLUTE_ERR_UNSUPPORTED,
                   "%s: K=%d at split %d needs %zu B of LDS (limit %d)", who, K, split,
                   plan->lds_bytes, kLdsPerCU);
     plan->grid_x = col;
+    plan->threads = waves * 64;
     plan->total_tickets = ticket;
-    int max_slots = 0;
-    for (int i = 0; i < count; ++i)
-        if (p.seg[i].nslots > max_slots) max_slots = p.seg[i].nslots;
-    plan->ws_floats = (size_t)max_slots * p.p_stride;
+    plan->p_floats = split > 1 ? (size_t)split * p.p_stride : 0;
+    plan->xb_floats = xb_off;
+    plan->xrot_halves = xrot_off;
     plan->lut_bf16 = lut_bf16;
     return FLUTE_OK;
 }
 
-template <bool BF16>
+template <bool BF16, int BFIX>
 flute_status launch_typed(Plan &plan, hipStream_t stream) {
-    static size_t attr_bytes = 0;
-    if (plan.lds_bytes > attr_bytes) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv_kernel<BF16>,
+    static bool attr_done = false;
+    if (!attr_done) {
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv_kernel<BF16, BFIX>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
                                             (int)kLdsPerCU));
-        attr_bytes = kLdsPerCU;
+        attr_done = true;
     }
+#ifdef FLUTE_GEMV_TRACE
+    {
+        const char *e = std::getenv("FLUTE_GEMV_TRACE_PTR");
+        plan.p.trace = e ? (unsigned long long *)std::strtoull(e, nullptr, 0) : nullptr;
+    }
+#endif
     dim3 grid(plan.grid_x, plan.p.split);
-    hipLaunchKernelGGL(gemv_kernel<BF16>, grid, dim3(kGemvThreads), plan.lds_bytes, stream, plan.p);
+    hipLaunchKernelGGL((gemv_kernel<BF16, BFIX>), grid, dim3(plan.threads), plan.lds_bytes, stream,
+                       plan.p);
     FLUTE_HIP_CHECK(hipGetLastError());
     return FLUTE_OK;
 }
 
-flute_status launch(Plan &plan, hipStream_t stream) {
-    bool need_ws = false;
-    for (int i = 0; i < kGemvMaxSegs; ++i) need_ws |= plan.p.seg[i].arrivals > 1;
-    if (need_ws) {
-        flute_status st = get_workspace(plan.ws_floats, (size_t)plan.total_tickets, stream,
-                                        &plan.p.P, &plan.p.tickets);
-        if (st != FLUTE_OK) return st;
+template <bool BF16>
+flute_status launch_width(Plan &plan, hipStream_t stream) {
+    // one width for the whole launch -> the instantiation specialised for it
+    int bits = plan.p.seg[0].st[0].bits;
+    for (int i = 0; i < plan.p.nsegs; ++i)
+        for (int st = 0; st < plan.p.seg[i].nstreams; ++st)
+            if (plan.p.seg[i].st[st].bits != bits) bits = 0;
+    switch (bits) {
+        case 4: return launch_typed<BF16, 4>(plan, stream);
+        case 3: return launch_typed<BF16, 3>(plan, stream);
+        case 2: return launch_typed<BF16, 2>(plan, stream);
+        case 1: return launch_typed<BF16, 1>(plan, stream);
+        default: return launch_typed<BF16, 0>(plan, stream);
     }
-    return plan.lut_bf16 ? launch_typed<true>(plan, stream) : launch_typed<false>(plan, stream);
+}
+
+flute_status launch(Plan &plan, int act_dtype, hipStream_t stream) {
+    if (plan.p_floats || plan.npre) {
+        const size_t xb_pad = (plan.xb_floats + 3) & ~(size_t)3;
+        const size_t floats = plan.p_floats + xb_pad + (plan.xrot_halves + 1) / 2 + 64;
+        float *base = nullptr;
+        int *tickets = nullptr;
+        flute_status st = get_workspace(floats, (size_t)plan.total_tickets + 1, stream, &base,
+                                        &tickets);
+        if (st != FLUTE_OK) return st;
+        plan.p.P = base;
+        plan.p.tickets = tickets;
+        float *xb_base = base + plan.p_floats;
+        uint16_t *xrot_base = (uint16_t *)(xb_base + xb_pad);
+        for (int i = 0; i < plan.npre; ++i) {
+            const Plan::Pre &pre = plan.pre[i];
+            const uint16_t *xin = plan.p.x;
+            if (pre.signs) {
+                uint16_t *xr = xrot_base + pre.xrot_off;
+                st = flute_fht(plan.p.x, pre.signs, pre.awq, xr, 1, plan.p.K, act_dtype, 0,
+                               plan.rot_block, stream);
+                if (st != FLUTE_OK) return st;
+                xin = xr;
+                plan.p.seg[pre.seg].xsrc = xr;
+            }
+            float *xb = xb_base + pre.xb_off;
+            hipLaunchKernelGGL(residual_coeff_kernel, dim3(pre.R), dim3(256), 0, stream, xin,
+                               pre.resB, xb, plan.p.K, plan.p.act_bf16);
+            FLUTE_HIP_CHECK(hipGetLastError());
+            plan.p.seg[pre.seg].xb = xb;
+        }
+    }
+    return plan.lut_bf16 ? launch_width<true>(plan, stream) : launch_width<false>(plan, stream);
 }
 
 }  // namespace
@@ -216,10 +327,9 @@ flute_status flute_gemv(const flute_linear *w, const void *x, void *y, int act_d
                         void *stream) {
     Plan plan;
     void *outs[1] = {y};
-    flute_status st = make_plan(w, 1, x, outs, act_dtype, split, 0,
-                                (w && w->signs) ? w->rot_block : 0, "flute_gemv", &plan);
+    flute_status st = make_plan(w, 1, x, outs, act_dtype, split, 0, "flute_gemv", &plan);
     if (st != FLUTE_OK) return st;
-    return launch(plan, (hipStream_t)stream);
+    return launch(plan, act_dtype, (hipStream_t)stream);
 }
 
 flute_status flute_gemv_mlp(const flute_linear *gate, const flute_linear *up, const void *x,
@@ -228,9 +338,9 @@ flute_status flute_gemv_mlp(const flute_linear *gate, const flute_linear *up, co
     flute_linear segs[2] = {*gate, *up};
     void *outs[2] = {h, h};
     Plan plan;
-    flute_status st = make_plan(segs, 2, x, outs, act_dtype, split, 1, 0, "flute_gemv_mlp", &plan);
+    flute_status st = make_plan(segs, 2, x, outs, act_dtype, split, 1, "flute_gemv_mlp", &plan);
     if (st != FLUTE_OK) return st;
-    return launch(plan, (hipStream_t)stream);
+    return launch(plan, act_dtype, (hipStream_t)stream);
 }
 
 flute_status flute_gemv_multi(const flute_linear *segs, int count, const void *x,
@@ -238,9 +348,9 @@ flute_status flute_gemv_multi(const flute_linear *segs, int count, const void *x
     FLUTE_REQUIRE(segs && outs, FLUTE_ERR_INVALID, "flute_gemv_multi: NULL argument");
     Plan plan;
     flute_status st =
-        make_plan(segs, count, x, outs, act_dtype, split, 0, 0, "flute_gemv_multi", &plan);
+        make_plan(segs, count, x, outs, act_dtype, split, 0, "flute_gemv_multi", &plan);
     if (st != FLUTE_OK) return st;
-    return launch(plan, (hipStream_t)stream);
+    return launch(plan, act_dtype, (hipStream_t)stream);
 }
 
 flute_status flute_mlp_block(const flute_linear *gate, const flute_linear *up,
@@ -256,15 +366,17 @@ flute_status flute_mlp_block(const flute_linear *gate, const flute_linear *up,
 
 int flute_pick_split(int N, int K) {
     if (N <= 0 || K <= 0 || N % 128 || K % 64) return 1;
-    return pick_split_tiles(N / 128, K / 64);
+    int rw, split, waves;
+    choose_shape(N, K / 64, 0, &rw, &split, &waves);
+    return split;
 }
 
 int64_t flute_gemv_lds_bytes(const flute_linear *w, int split) {
     Plan plan;
     char dummy_x = 0, dummy_y = 0;
     void *outs[1] = {&dummy_y};
-    if (make_plan(w, 1, &dummy_x, outs, FLUTE_F16 + (w && w->lut_dtype == FLUTE_BF16), split, 0, 0,
-                  "flute_gemv_lds_bytes", &plan) != FLUTE_OK)
+    if (make_plan(w, 1, &dummy_x, outs, (w && w->lut_dtype == FLUTE_BF16) ? FLUTE_BF16 : FLUTE_F16,
+                  split, 0, "flute_gemv_lds_bytes", &plan) != FLUTE_OK)
         return 0;
     return (int64_t)plan.lds_bytes;
 }

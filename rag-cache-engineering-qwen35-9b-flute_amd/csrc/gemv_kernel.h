@@ -1,34 +1,36 @@
 // M = 1 LUT GEMV for gfx950 (wave64), the decode kernel of the idxN layer.
 //
-// Work decomposition.  The unit of work is one STREAM of one weight, one
-// 128-row tile t, one K-split s:  workgroup (x = tile column, y = s), 256
-// threads = 4 wavefronts.  Wavefront u owns QUARTER u of every 64-k tile of
-// the split: the 16 consecutive thread-chunks [16u, 16u+16) of the idxN tile,
-// which are 256*b contiguous bytes.  Lane L reads the 4*b bytes at L*4*b of
-// that quarter — one fully coalesced load per tile per wavefront — and those
-// bytes are exactly quarter kt = L & 3 of chunk c = 16u + (L >> 2), i.e.
+// Ownership.  A workgroup OWNS a slice of RW output rows of one 128-row tile
+// (RW = 8, 16 or 32: 1, 2 or 4 of the tile's sixteen 8-row chunk groups) and,
+// when K is split, one K range.  Its wavefronts all work on the same rows and
+// divide the 64-k tiles of the range between them; a workgroup runs every
+// stream that feeds its rows (one or two streams of a weight; gate and up of a
+// merged MLP) one after the other, so without a K split no partial result ever
+// leaves the workgroup.
 //
-//     rows  n = t*128 + (u>>1)*64 + v*16 + d*8 + 4*(u&1) + (L>>4)   (v<4, d<2)
-//     cols  k = g*64 + (L&3)*16 + 2*((L>>2)&3) + 8*s2  and k+1     (s2<2)
+// Reading the blob (flute_extended/idxN.py:37-55 upstream).  In a tile of
+// 1024*b bytes, chunk group cg = (wx, r8) is the 64*b contiguous bytes of the
+// four chunks i = 0..3 that cover rows wx*64 + v*16 + d*8 + r8 (v<4, d<2).
+// A lane reads 4*b bytes: quarter kt of one chunk, i.e. 16 k-pairs
+// q = v*4 + d*2 + s2 of columns kt*16 + 2*i + 8*s2 (+1).  With LPG = 2*RW lanes
+// per 64-k tile, lane l = (cg_local, i, kt) and a wavefront load covers 64/LPG
+// tiles at once, each as one contiguous run of LPG*4*b bytes.  A lane therefore
+// keeps 8 fp32 row accumulators (v, d) for its whole K share; the lanes that
+// share rows are folded once at the end (DPP inside 16 lanes, then across).
 //
-// so a lane keeps 8 fp32 row accumulators for the whole K range and the 16
-// lanes L&15 that share a row are folded once at the end with DPP.
+// Dequantisation.  The group's LUT (2^b 16-bit values) is expanded once per
+// workgroup into a paired table in LDS indexed by a whole packed byte (b = 4:
+// byte -> {W[k], W[k+1]}; b = 2: byte -> 4 values; b = 1: byte -> 8 values;
+// b = 3: 6-bit pair field -> 2 values).  Every entry is replicated across a
+// power-of-two stride so that each lane reads its own bank: one conflict-free
+// ds_read per lookup whatever the codes are.  With a 256-byte stride the address
+// is {replica byte, code byte} and is formed by a single v_perm_b32.  A pair
+// feeds v_dot2_f32_f16 / v_dot2_f32_bf16 against the matching activation pair:
+// 2 MACs per instruction, fp32 accumulate.
 //
-// Dequantisation.  The per-group LUT (2^b 16-bit values) is expanded once per
-// workgroup into a paired table in LDS that is indexed by a whole packed byte
-// (b = 4: byte -> {W[k], W[k+1]}; b = 2: byte -> 4 values; b = 1: byte -> 8
-// values; b = 3: 6-bit pair field -> 2 values).  Every entry is replicated
-// across a power-of-two stride so that each lane reads its own bank: a lookup
-// is one ds_read with no bank conflicts whatever the codes are.  With a 256-byte
-// stride the address is {slot byte, code byte} and is formed by one v_perm_b32.
-// A looked-up pair feeds v_dot2_f32_f16 / v_dot2_f32_bf16 against the matching
-// activation pair: 2 MACs per instruction, fp32 accumulate.
-//
-// Split-K.  Row partials of every (stream, split) slot go to a workspace
-// P[slot][column]; the last workgroup to arrive at an output tile (a ticket
-// counter per tile) folds the slots in fixed order, adds the low-rank residual
-// and the bias in fp32, applies SiLU*mul for the merged gate/up mode, rounds
-// once and resets the ticket, so the launch is deterministic and replayable.
+// K split (narrow N only).  Row partials go to a workspace through
+// device-coherent stores; the last workgroup to take a ticket for a row slice
+// folds them in fixed order.  Deterministic and replayable: tickets return to 0.
 #pragma once
 
 #include "common.h"
@@ -36,59 +38,66 @@
 
 namespace flute {
 
-constexpr int kGemvThreads = 256;
-constexpr int kGemvMaxJobs = 8;
+constexpr int kGemvMaxThreads = 512;
 constexpr int kGemvMaxSegs = 4;
 constexpr int kGemvMaxRank = 256;
-constexpr int kPrefetch = 8;          // 64-k tiles of index data in flight per lane
 
-struct GemvJob {            // one stream of one weight
+struct GemvStream {
     const uint8_t *q;       // idxN blob
-    const uint16_t *lut;    // [rows, 2^bits]
-    int tile0;              // first grid column of this job
-    int ntiles;             // N / 128
+    const uint16_t *lut;    // [lut_rows, 2^bits]
     int bits;
-    int seg;
     int es;                 // log2(LDS bytes between consecutive table entries)
-    int slot0;              // first partial-sum slot of this stream
 };
 
 struct GemvSeg {            // one weight
-    const uint16_t *resB;   // (R, K) or null
+    GemvStream st[2];
     const uint16_t *resA;   // (N, R) or null
     const uint16_t *bias;   // (N,) or null
+    const float *xb;        // (R,) residual coefficients x . resB[r], fp32, or null
+    const uint16_t *xsrc;   // (K,) this weight's own input row, or null for the shared one
     const float *signs;     // (K,) or null: rotate the input first
     const float *awq;       // (K,) or null
     uint16_t *out;          // (N,)
+    int nstreams;
     int N;
     int R;
     int gs;
     int lut_rows;
-    int nslots;             // partial-sum slots of this weight (streams * split)
-    int arrivals;           // workgroups that must arrive before an output tile is finished
+    int col0;               // first grid column (row slice) of this weight
     int n0;                 // first column of this weight in a partial-sum row
-    int r0;                 // first residual column of this weight
     int ticket0;            // first ticket of this weight
 };
 
 struct GemvParams {
-    GemvJob job[kGemvMaxJobs];
     GemvSeg seg[kGemvMaxSegs];
     const uint16_t *x;      // (K,) activations
-    float *P;               // partial sums: [slot][p_stride]
+    float *P;               // partial sums: [split][p_stride]
     int *tickets;
-    int njobs;
+    int nsegs;
     int K;
     int split;
     int gs_tiles;           // 64-k tiles per split
+    int lpg_log2;           // log2(lanes per 64-k tile) = log2(2 * RW): 4, 5 or 6
     int p_stride;           // floats per partial-sum row
     int silu_mul;           // 1: out = silu(seg 0) * seg 1, written to seg[0].out
     int act_bf16;           // activations, residual, bias and outputs are bf16
     int fht_block;          // > 0: equal rotation blocks of this many columns
     int lds_x;              // LDS byte offsets
     int lds_red;
-    int lds_xb;
+#ifdef FLUTE_GEMV_TRACE
+    unsigned long long *trace;   // [workgroup][8] timestamps, development builds only
+#endif
 };
+
+#ifdef FLUTE_GEMV_TRACE
+#define FLUTE_TRACE(slot)                                                              \
+    do {                                                                               \
+        if (p.trace && threadIdx.x == 0)                                               \
+            p.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8 + (slot)] = wall_clock64(); \
+    } while (0)
+#else
+#define FLUTE_TRACE(slot) do {} while (0)
+#endif
 
 // ---- small device helpers ---------------------------------------------------
 
@@ -96,6 +105,16 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
     int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
     return v + __builtin_bit_cast(float, moved);
+}
+
+// Workspace traffic between workgroups goes through device-scope atomic
+// stores and loads: they bypass the non-coherent cache levels (each XCD has its
+// own L2), so no cache write-back or invalidate is needed around the ticket.
+__device__ __forceinline__ void ws_store(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ws_load(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Sum over the 16 lanes of a DPP row; every lane of the row ends with the total.
@@ -107,14 +126,7 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-    v = row16_sum(v);
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
-}
-
-// Table geometry per width: entries, bytes per entry.
+// Table geometry per width: entries, log2(bytes per entry).
 template <int B> struct TableShape;
 template <> struct TableShape<4> { static constexpr int kEntries = 256, kEntryLog2 = 2; };
 template <> struct TableShape<3> { static constexpr int kEntries = 64,  kEntryLog2 = 2; };
@@ -132,41 +144,13 @@ __device__ __forceinline__ uint32_t table_dword(const uint16_t *lut, int e, int 
     return (uint32_t)lut[c0] | ((uint32_t)lut[c1] << 16);
 }
 
-// Expand `ngrp` LUT rows into replicated paired tables at tab (LDS).  Table of
-// group q starts at q * (kEntries << es); entry e at e << es; the entry repeats
-// every kEntryBytes inside its stride.  A thread owns one (group, entry) at a
-// time and walks the replicas starting at a lane-dependent one, so that the 64
-// lanes of a wavefront write 64 different banks.
-template <int B>
-__device__ __forceinline__ void build_tables(uint8_t *tab, const uint16_t *lut_rows, int ngrp,
-                                             int es, int tid) {
-    constexpr int E = TableShape<B>::kEntries;
-    constexpr int EL = TableShape<B>::kEntryLog2;
-    constexpr int EDW = 1 << (EL - 2);              // dwords per entry
-    const int nrep = 1 << (es - EL);                // replicas per entry
-    for (int item = tid; item < ngrp * E; item += kGemvThreads) {
-        const int q = item / E, e = item % E;
-        const uint16_t *lut = lut_rows + ((size_t)q << B);
-        uint32_t val[EDW];
-#pragma unroll
-        for (int s = 0; s < EDW; ++s) val[s] = table_dword<B>(lut, e, s);
-        uint8_t *ent = tab + (size_t)q * (E << es) + ((size_t)e << es);
-        for (int r = 0; r < nrep; ++r) {
-            const int rep = (r + tid) & (nrep - 1);
-            uint32_t *dst = (uint32_t *)(ent + (rep << EL));
-#pragma unroll
-            for (int s = 0; s < EDW; ++s) dst[s] = val[s];
-        }
-    }
-}
-
-// One quarter-tile (4*B bytes of this lane) against the activation pairs xa
+// One quarter-chunk (4*B bytes of this lane) against the activation pairs xa
 // (s2 = 0) and xb (s2 = 1).  lane_off[v] = table base of row block v plus this
 // lane's replica offset.
 template <int B, bool BF16, bool PERM>
-__device__ __forceinline__ void consume_tile(const uint32_t (&w)[B], uint32_t xa, uint32_t xb,
-                                             const uint8_t *lds, const uint32_t (&lane_off)[4],
-                                             int es, float (&acc)[8]) {
+__device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t xa, uint32_t xb,
+                                                const uint8_t *lds, const uint32_t (&lane_off)[4],
+                                                int es, float (&acc)[8]) {
     if constexpr (B == 4) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -215,7 +199,7 @@ __device__ __forceinline__ void consume_tile(const uint32_t (&w)[B], uint32_t xa
             acc[v * 2 + 1] = dot2<BF16>(e.z, xa, acc[v * 2 + 1]);
             acc[v * 2 + 1] = dot2<BF16>(e.w, xb, acc[v * 2 + 1]);
         }
-    } else {                                        // B == 3: 24-bit group per v
+    } else {                                        // B == 3: one 24-bit group per v
         const uint32_t grp[4] = {
             w[0],
             __builtin_amdgcn_alignbit(w[1], w[0], 24),
@@ -250,37 +234,68 @@ __device__ __forceinline__ void load_quarter(uint32_t (&w)[B], const uint8_t *p)
     }
 }
 
-// Stage the activation slice [k0, k0 + kc) into LDS as 16-bit values of the
-// compute type (the LUT's type).  With signs, the rotation of every segment
-// that overlaps the slice is computed first in the fp32 scratch (which aliases
-// the not-yet-built tables), rounded to the activation type exactly as the
-// standalone rotation kernel rounds, and only then converted.
+// Eight consecutive activations (16 bytes) as floats.
+__device__ __forceinline__ void load_act8(const uint16_t *x, int k, int is_bf16, float (&f)[8]) {
+    const uint4 v = *(const uint4 *)(x + k);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint16_t lo = (uint16_t)(w[j] & 0xffffu), hi = (uint16_t)(w[j] >> 16);
+        f[2 * j] = is_bf16 ? bf2f(lo) : h2f(lo);
+        f[2 * j + 1] = is_bf16 ? bf2f(hi) : h2f(hi);
+    }
+}
+
+// Eight raw activations -> eight values of the compute type.
 template <bool BF16>
-__device__ void stage_x(const GemvParams &p, const GemvSeg &sg, uint8_t *lds, int k0, int kc,
-                        int tid) {
+__device__ __forceinline__ uint4 to_compute_type(uint4 v, int act_bf16) {
+    if (act_bf16 && !BF16) {                       // bf16 activations, fp16 compute type
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            w[q] = (uint32_t)f2h(bf2f((uint16_t)(w[q] & 0xffffu))) |
+                   ((uint32_t)f2h(bf2f((uint16_t)(w[q] >> 16))) << 16);
+        v = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    return v;
+}
+
+// Stage the activation slice [k0, k0 + kc) into LDS as 16-bit values of the
+// compute type (the LUT's type), 16 bytes per thread per step so that the whole
+// slice is one round trip to memory.  With signs, the rotation of every segment
+// that overlaps the slice is computed first in the fp32 scratch at the start of
+// LDS (where the tables are built afterwards), rounded to the activation type
+// exactly as the standalone rotation kernel rounds, and only then converted.
+// Ends with the slice complete and the scratch free (barrier included).
+template <bool BF16>
+__device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *signs,
+                        const float *awq, uint8_t *lds, int k0, int kc, int tid, int nthreads) {
     uint16_t *xs = (uint16_t *)(lds + p.lds_x);
-    if (sg.signs == nullptr) {
-        for (int j = tid; j < kc; j += kGemvThreads) {
-            const float f = load_act(p.x, k0 + j, p.act_bf16);
-            xs[j] = BF16 ? f2bf(f) : f2h(f);
-        }
+    if (signs == nullptr) {
+        for (int j = tid * 8; j < kc; j += nthreads * 8)
+            *(uint4 *)(xs + j) = to_compute_type<BF16>(*(const uint4 *)(x + k0 + j), p.act_bf16);
+        __syncthreads();
         return;
     }
     float *buf = (float *)lds;
     if (p.fht_block > 0) {
         // equal blocks: the slice is a whole number of blocks
-        for (int j = tid; j < kc; j += kGemvThreads) {
-            float f = load_act(p.x, k0 + j, p.act_bf16);
-            if (sg.awq) f *= sg.awq[k0 + j];
-            buf[fht_slot(j)] = f;
+        for (int j = tid * 8; j < kc; j += nthreads * 8) {
+            float f[8];
+            load_act8(x, k0 + j, p.act_bf16, f);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                if (awq) f[q] *= awq[k0 + j + q];
+                buf[fht_slot(j + q)] = f[q];
+            }
         }
         __syncthreads();
         const int nst = 31 - __builtin_clz((unsigned)p.fht_block);
-        fht_lds(buf, kc, nst, tid, kGemvThreads);
+        fht_lds(buf, kc, nst, tid, nthreads);
         const float inv = inv_sqrt_pow2(nst);
-        for (int j = tid; j < kc; j += kGemvThreads) {
-            float t = buf[fht_slot(j)] * sg.signs[k0 + j] * inv;
-            if (sg.awq) t = t / sg.awq[k0 + j];
+        for (int j = tid; j < kc; j += nthreads) {
+            float t = buf[fht_slot(j)] * signs[k0 + j] * inv;
+            if (awq) t = t / awq[k0 + j];
             const uint16_t a = round_act(t, p.act_bf16);
             const float back = p.act_bf16 ? bf2f(a) : h2f(a);
             xs[j] = BF16 ? f2bf(back) : f2h(back);
@@ -294,17 +309,21 @@ __device__ void stage_x(const GemvParams &p, const GemvSeg &sg, uint8_t *lds, in
         const int b = 1 << nst;
         const int lo = max(off, k0), hi = min(off + b, k0 + kc);
         if (lo < hi) {                             // uniform across the workgroup
-            for (int j = tid; j < b; j += kGemvThreads) {
-                float f = load_act(p.x, off + j, p.act_bf16);
-                if (sg.awq) f *= sg.awq[off + j];
-                buf[fht_slot(j)] = f;
+            for (int j = tid * 8; j < b; j += nthreads * 8) {
+                float f[8];
+                load_act8(x, off + j, p.act_bf16, f);
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    if (awq) f[q] *= awq[off + j + q];
+                    buf[fht_slot(j + q)] = f[q];
+                }
             }
             __syncthreads();
-            fht_lds(buf, b, nst, tid, kGemvThreads);
+            fht_lds(buf, b, nst, tid, nthreads);
             const float inv = inv_sqrt_pow2(nst);
-            for (int k = lo + tid; k < hi; k += kGemvThreads) {
-                float t = buf[fht_slot(k - off)] * sg.signs[k] * inv;
-                if (sg.awq) t = t / sg.awq[k];
+            for (int k = lo + tid; k < hi; k += nthreads) {
+                float t = buf[fht_slot(k - off)] * signs[k] * inv;
+                if (awq) t = t / awq[k];
                 const uint16_t a = round_act(t, p.act_bf16);
                 const float back = p.act_bf16 ? bf2f(a) : h2f(a);
                 xs[k - k0] = BF16 ? f2bf(back) : f2h(back);
@@ -316,212 +335,418 @@ __device__ void stage_x(const GemvParams &p, const GemvSeg &sg, uint8_t *lds, in
     }
 }
 
-// Finish one output row: fold the partial-sum slots in ascending order, add the
-// residual and the bias.  Everything in fp32.
-__device__ __forceinline__ float fold_row(const GemvParams &p, const GemvSeg &sg, int n,
-                                          bool from_workspace, float own) {
-    float y;
-    if (from_workspace) {
-        y = 0.0f;
-        for (int s = 0; s < sg.nslots; ++s)
-            y += __hip_atomic_load(p.P + (size_t)s * p.p_stride + sg.n0 + n, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-    } else {
-        y = own;
+// Geometry of this lane inside its workgroup, fixed for the whole kernel.
+struct LaneGeom {
+    int tid, nthreads, w, nwaves, L;
+    int gsub;        // which of the 64/LPG tiles of a wavefront load this lane reads
+    int l;           // lane within the tile: (cg_local, i, kt)
+    int t;           // 128-row tile
+    int cg0;         // first chunk group of the row slice
+    int cg;          // this lane's chunk group
+    int g_lo;        // first 64-k tile of the K range
+    int units;       // wavefront loads covering the K range
+    int gpi;         // 64-k tiles per wavefront load
+};
+
+// Per-lane state of one stream pass between its phases.
+template <int B>
+struct StreamRegs {
+    static constexpr int kPrefetch = B == 4 ? 4 : (B == 3 ? 5 : 8);   // loads in flight per lane
+    static constexpr int kEDW = 1 << (TableShape<B>::kEntryLog2 - 2);
+    uint32_t q[kPrefetch][B];
+    uint32_t val[kEDW];      // this thread's table entry (fast path)
+    const uint8_t *qrow;
+    uint32_t lane0, step;
+    int my_units;
+    int grp0, ngrp;
+    bool fast_table;         // one (group, entry) item per thread: values already in val
+};
+
+// Phase 1 - global loads only: the first index bytes of this lane and the LUT
+// values of the table entry this thread will write.  Nothing here waits.
+template <int B>
+__device__ __forceinline__ void stream_issue(const GemvParams &p, const GemvSeg &sg,
+                                             const GemvStream &st, const LaneGeom &gm,
+                                             StreamRegs<B> &r) {
+    constexpr int E = TableShape<B>::kEntries;
+    constexpr int PF = StreamRegs<B>::kPrefetch;
+    const int G = p.K >> 6;
+    // uniform 64-bit base of this tile row's K range + a 32-bit lane offset (a
+    // tile row is at most 4 MB)
+    r.qrow = st.q + ((size_t)gm.t * G + gm.g_lo) * (1024 * B);
+    const uint32_t unit_bytes = (uint32_t)gm.gpi * (1024 * B);
+    r.lane0 = (uint32_t)gm.gsub * (1024 * B) + (uint32_t)gm.cg0 * (64 * B) +
+              (uint32_t)gm.l * (4 * B) + (uint32_t)gm.w * unit_bytes;
+    r.step = (uint32_t)gm.nwaves * unit_bytes;
+    r.my_units = gm.units > gm.w ? (gm.units - gm.w + gm.nwaves - 1) / gm.nwaves : 0;
+    const int gs = sg.gs;
+    const int ngrp_all = gs >= 128 ? 1 : 128 / gs;
+    r.grp0 = min((gm.t * 128) / gs, sg.lut_rows - 1);
+    r.ngrp = min(ngrp_all, sg.lut_rows - r.grp0);
+    const int items = r.ngrp * E;
+    r.fast_table = items <= gm.nthreads;
+    if (r.fast_table) {
+        const int item = gm.tid % items;
+        const uint16_t *lut = st.lut + ((size_t)(r.grp0 + item / E) << B);
+#pragma unroll
+        for (int s = 0; s < StreamRegs<B>::kEDW; ++s) r.val[s] = table_dword<B>(lut, item % E, s);
     }
-    return y;
+#pragma unroll
+    for (int n = 0; n < PF; ++n) {
+#pragma unroll
+        for (int j = 0; j < B; ++j) r.q[n][j] = 0u;
+        if (n < r.my_units) load_quarter<B>(r.q[n], r.qrow + (r.lane0 + (uint32_t)n * r.step));
+    }
 }
 
-template <int B, bool BF16>
-__device__ void gemv_body(const GemvParams &p, const GemvJob &jb, const GemvSeg &sg,
-                          uint8_t *lds) {
-    const int tid = threadIdx.x;
-    const int u = tid >> 6;                         // quarter of the tile
-    const int L = tid & 63;
-    const int t = blockIdx.x - jb.tile0;
-    const int s = blockIdx.y;
-    const int G = p.K >> 6;
-    const int g0 = s * p.gs_tiles;
-    const int k0 = g0 * 64, kc = p.gs_tiles * 64;
-
-    // ---- issue the first index loads before the prologue: up to kPrefetch tiles
-    //      of this lane are in flight at any time -------------------------------
-    const uint8_t *qbase = jb.q + ((size_t)t * G + g0) * (1024 * B) + u * (256 * B) + L * (4 * B);
-    uint32_t q[kPrefetch][B];
-#pragma unroll
-    for (int i = 0; i < kPrefetch; ++i) {
-#pragma unroll
-        for (int j = 0; j < B; ++j) q[i][j] = 0u;
-        if (i < p.gs_tiles) load_quarter<B>(q[i], qbase + (size_t)i * (1024 * B));
-    }
-
-    // ---- activations (and rotation) into LDS ----------------------------------
-    stage_x<BF16>(p, sg, lds, k0, kc, tid);
-    __syncthreads();
-
-    // ---- residual partials of this K slice: only stream 1 carries them --------
-    const bool direct = (sg.arrivals == 1);
-    float *xB = (float *)(lds + p.lds_xb);
-    if (sg.R > 0 && jb.slot0 == 0) {
-        const uint16_t *xs = (const uint16_t *)(lds + p.lds_x);
-        for (int r = u; r < sg.R; r += 4) {
-            const uint16_t *brow = sg.resB + (size_t)r * p.K + k0;
-            float part = 0.0f;
-            for (int k = L; k < kc; k += 64) {
-                const float xv = BF16 ? bf2f(xs[k]) : h2f(xs[k]);
-                part = fmaf(xv, p.act_bf16 ? bf2f(brow[k]) : h2f(brow[k]), part);
-            }
-            part = wave_sum(part);
-            if (L == 0) {
-                if (direct) xB[r] = part;
-                else p.P[(size_t)s * p.p_stride + sg.r0 + r] = part;
-            }
-        }
-    }
-
-    // ---- paired tables of the groups this tile touches ------------------------
+// Phase 2 - expand the LUT rows into replicated paired tables at the start of
+// LDS.  Table of group q starts at q * (E << es); entry e at e << es and repeats
+// every entry-size bytes inside its stride.  A thread owns one (group, entry)
+// and a share of its replicas; the walk starts at a lane-dependent replica so
+// that a wavefront writes 64 different banks.
+template <int B>
+__device__ __forceinline__ void stream_tables(const GemvStream &st, const LaneGeom &gm,
+                                              uint8_t *lds, const StreamRegs<B> &r) {
     constexpr int E = TableShape<B>::kEntries;
     constexpr int EL = TableShape<B>::kEntryLog2;
-    const int gs = sg.gs;
-    const int ngrp = gs >= 128 ? 1 : 128 / gs;
-    const int grp0 = (t * 128) / gs;
-    // rows past the last LUT row reuse it (scripts/palettized_modules.py:155-156 upstream)
-    const int grp0c = min(grp0, sg.lut_rows - 1);
-    build_tables<B>(lds, jb.lut + ((size_t)grp0c << B), min(ngrp, sg.lut_rows - grp0c), jb.es, tid);
+    constexpr int EDW = StreamRegs<B>::kEDW;
+    const int es = st.es;
+    const int items = r.ngrp * E;
+    const int nrep = 1 << (es - EL);
+    int shares = gm.nthreads / items;
+    if (shares < 1) shares = 1;
+    if (shares > nrep) shares = nrep;
+    const int per = nrep / shares;
+    for (int it = gm.tid; it < items * shares; it += gm.nthreads) {
+        const int item = it % items, share = it / items;
+        const int qg = item / E, e = item % E;
+        uint32_t val[EDW];
+        if (r.fast_table) {
+#pragma unroll
+            for (int s = 0; s < EDW; ++s) val[s] = r.val[s];
+        } else {
+            const uint16_t *lut = st.lut + ((size_t)(r.grp0 + qg) << B);
+#pragma unroll
+            for (int s = 0; s < EDW; ++s) val[s] = table_dword<B>(lut, e, s);
+        }
+        uint8_t *ent = lds + (size_t)qg * (E << es) + ((size_t)e << es);
+        for (int k = 0; k < per; ++k) {
+            const int rep = share * per + ((k + gm.tid) & (per - 1));
+            uint32_t *dst = (uint32_t *)(ent + (rep << EL));
+#pragma unroll
+            for (int s = 0; s < EDW; ++s) dst[s] = val[s];
+        }
+    }
+}
 
-    const int es = jb.es;
+// Phase 3 - stream the index bytes of this lane against the staged activations.
+template <int B, bool BF16>
+__device__ __forceinline__ void stream_loop(const GemvParams &p, const GemvSeg &sg,
+                                            const GemvStream &st, const LaneGeom &gm,
+                                            uint8_t *lds, StreamRegs<B> &r, float (&acc)[8]) {
+    constexpr int E = TableShape<B>::kEntries;
+    constexpr int EL = TableShape<B>::kEntryLog2;
+    constexpr int PF = StreamRegs<B>::kPrefetch;
+    const int es = st.es;
+    const int gs = sg.gs;
     const int slot_mask = (1 << (es - EL)) - 1;
     uint32_t lane_off[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-        const int row_local = (u >> 1) * 64 + v * 16;
-        int q = gs >= 128 ? 0 : row_local / gs;
-        q = min(q, sg.lut_rows - 1 - grp0c);
-        lane_off[v] = (uint32_t)(q * (E << es) + ((L & slot_mask) << EL));
+        const int row_local = (gm.cg >> 3) * 64 + v * 16;
+        int qg = gs >= 128 ? 0 : row_local / gs;
+        qg = min(qg, r.ngrp - 1);
+        lane_off[v] = (uint32_t)(qg * (E << es) + ((gm.L & slot_mask) << EL));
     }
-    __syncthreads();
-
-    // ---- K loop ---------------------------------------------------------------
-    float acc[8];
-#pragma unroll
-    for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
     const uint32_t *xs32 = (const uint32_t *)(lds + p.lds_x);
-    const int xi = (L & 3) * 8 + ((L >> 2) & 3);   // kt*8 + i
+    const int xi = gm.gsub * 32 + (gm.l & 3) * 8 + ((gm.l >> 2) & 3);   // + unit * gpi * 32
     const bool perm = (es == 8);
-    for (int gb = 0; gb < p.gs_tiles; gb += kPrefetch) {
+    for (int nb = 0; nb < r.my_units; nb += PF) {
 #pragma unroll
-        for (int i = 0; i < kPrefetch; ++i) {
-            const int g = gb + i;
-            if (g < p.gs_tiles) {                   // uniform
-                uint32_t w[B];
+        for (int n = 0; n < PF; ++n) {
+            const int m = nb + n;
+            if (m < r.my_units) {                   // uniform within the wavefront
+                uint32_t wq[B];
 #pragma unroll
-                for (int j = 0; j < B; ++j) w[j] = q[i][j];
-                if (g + kPrefetch < p.gs_tiles)
-                    load_quarter<B>(q[i], qbase + (size_t)(g + kPrefetch) * (1024 * B));
-                const uint32_t xa = xs32[g * 32 + xi];
-                const uint32_t xb = xs32[g * 32 + xi + 4];
+                for (int j = 0; j < B; ++j) wq[j] = r.q[n][j];
+                if (m + PF < r.my_units)
+                    load_quarter<B>(r.q[n], r.qrow + (r.lane0 + (uint32_t)(m + PF) * r.step));
+                const int xo = (gm.w + m * gm.nwaves) * gm.gpi * 32 + xi;
+                const uint32_t xa = xs32[xo];
+                const uint32_t xb = xs32[xo + 4];
                 if (B != 3 && perm)
-                    consume_tile<B, BF16, (B != 3)>(w, xa, xb, lds, lane_off, es, acc);
+                    consume_quarter<B, BF16, (B != 3)>(wq, xa, xb, lds, lane_off, es, acc);
                 else
-                    consume_tile<B, BF16, false>(w, xa, xb, lds, lane_off, es, acc);
+                    consume_quarter<B, BF16, false>(wq, xa, xb, lds, lane_off, es, acc);
             }
         }
     }
+}
 
-    // ---- fold the 16 lanes that share a row -----------------------------------
+// One stream pass whose loads were not issued ahead: all three phases in a row.
+// Ends with a barrier so that the table region may be rewritten.
+template <int B, bool BF16>
+__device__ void run_stream(const GemvParams &p, const GemvSeg &sg, const GemvStream &st,
+                           const LaneGeom &gm, uint8_t *lds, float (&acc)[8]) {
+    StreamRegs<B> r;
+    stream_issue<B>(p, sg, st, gm, r);
+    stream_tables<B>(st, gm, lds, r);
+    __syncthreads();
+    stream_loop<B, BF16>(p, sg, st, gm, lds, r, acc);
+    __syncthreads();
+}
+
+// BFIX != 0: every stream of the launch has this width (the common case, one
+// lean instantiation per width); BFIX == 0: widths are mixed and chosen per stream.
+template <bool BF16, int BFIX>
+__device__ __forceinline__ void run_stream_any(const GemvParams &p, const GemvSeg &sg,
+                                               const GemvStream &st, const LaneGeom &gm,
+                                               uint8_t *lds, float (&acc)[8]) {
+    if constexpr (BFIX != 0) {
+        run_stream<BFIX, BF16>(p, sg, st, gm, lds, acc);
+        return;
+    }
+    switch (st.bits) {
+        case 4: run_stream<4, BF16>(p, sg, st, gm, lds, acc); break;
+        case 3: run_stream<3, BF16>(p, sg, st, gm, lds, acc); break;
+        case 2: run_stream<2, BF16>(p, sg, st, gm, lds, acc); break;
+        default: run_stream<1, BF16>(p, sg, st, gm, lds, acc); break;
+    }
+}
+
+// Tile-local row of accumulator a of chunk group cg.
+__device__ __forceinline__ int row_of(int cg, int a) {
+    return (cg >> 3) * 64 + (a >> 1) * 16 + (a & 1) * 8 + (cg & 7);
+}
+
+template <bool BF16, int BFIX>
+__global__ void __launch_bounds__(kGemvMaxThreads, 4) gemv_kernel(const GemvParams p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+
+    // Read the weight descriptors straight from the kernel-argument segment
+    // (constant address space): a dynamic index then costs a scalar load with an
+    // offset instead of a select chain over every field of every descriptor.
+    const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
+    int si0 = 0;
+    if (!p.silu_mul) {
 #pragma unroll
-    for (int a = 0; a < 8; ++a) acc[a] = row16_sum(acc[a]);
-    float *red = (float *)(lds + p.lds_red);        // [128] row sums of this workgroup
-    if ((L & 15) == 0) {
+        for (int i = 1; i < kGemvMaxSegs; ++i)
+            if (i < p.nsegs && (int)blockIdx.x >= p.seg[i].col0) si0 = i;
+    }
+    const GemvSeg sg = kp->seg[si0];
+
+    LaneGeom gm;
+    gm.tid = threadIdx.x;
+    gm.nthreads = blockDim.x;
+    gm.w = gm.tid >> 6;
+    gm.nwaves = gm.nthreads >> 6;
+    gm.L = gm.tid & 63;
+    const int lpg = 1 << p.lpg_log2;
+    gm.gsub = gm.L >> p.lpg_log2;
+    gm.l = gm.L & (lpg - 1);
+    gm.gpi = 64 >> p.lpg_log2;
+    const int rw = lpg >> 1;                        // rows per workgroup
+    const int spt = 128 / rw;                       // row slices per tile
+    const int sl = (int)blockIdx.x - sg.col0;
+    gm.t = sl / spt;
+    gm.cg0 = (sl % spt) * (rw >> 3);
+    gm.cg = gm.cg0 + (gm.l >> 4);
+    const int s = blockIdx.y;
+    gm.g_lo = s * p.gs_tiles;
+    gm.units = p.gs_tiles / gm.gpi;
+    const int k0 = gm.g_lo * 64, kc = p.gs_tiles * 64;
+
+    float *red = (float *)(lds + p.lds_red);        // [2][nwaves][32] row sums
+    const int nout = p.silu_mul ? 2 : 1;
+    const float *staged_signs = nullptr, *staged_awq = nullptr;
+    const uint16_t *staged_x = nullptr;
+    bool staged = false;
+    // With one width for the whole launch, the very first pass issues its index
+    // and LUT loads BEFORE the activations are staged, so that the three kinds
+    // of loads travel together; later passes issue theirs when they start.
+    // Load order matters: activations, then LUT values, then index bytes, so that
+    // each consumer waits only for what was issued before it.
+    constexpr int BF = BFIX != 0 ? BFIX : 4;
+    constexpr int XV = 2;                           // 16-byte activation loads per thread
+    StreamRegs<BF> first;
+    uint4 xv[XV];
+    const uint16_t *x0 = sg.xsrc ? sg.xsrc : p.x;
+    const bool x_ahead = BFIX != 0 && sg.signs == nullptr;      // uniform
+    FLUTE_TRACE(0);
+    if (x_ahead) {
+#pragma unroll
+        for (int i = 0; i < XV; ++i) {
+            const int j = (i * gm.nthreads + gm.tid) * 8;
+            xv[i] = make_uint4(0u, 0u, 0u, 0u);
+            if (j < kc) xv[i] = *(const uint4 *)(x0 + k0 + j);
+        }
+    }
+    if constexpr (BFIX != 0) stream_issue<BF>(p, sg, sg.st[0], gm, first);
+    FLUTE_TRACE(1);
+
+    for (int so = 0; so < nout; ++so) {
+        const GemvSeg og = kp->seg[so == 1 ? 1 : si0];
+        const uint16_t *xin = og.xsrc ? og.xsrc : p.x;
+        if (so == 0 && x_ahead) {
+            uint16_t *xs = (uint16_t *)(lds + p.lds_x);
+#pragma unroll
+            for (int i = 0; i < XV; ++i) {
+                const int j = (i * gm.nthreads + gm.tid) * 8;
+                if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(xv[i], p.act_bf16);
+            }
+            for (int j = (XV * gm.nthreads + gm.tid) * 8; j < kc; j += gm.nthreads * 8)
+                *(uint4 *)(xs + j) = to_compute_type<BF16>(*(const uint4 *)(x0 + k0 + j), p.act_bf16);
+            // no barrier here: the one after the table build publishes both
+            staged = true;
+            staged_x = xin;
+            staged_signs = og.signs;
+            staged_awq = og.awq;
+        } else if (!staged || xin != staged_x || og.signs != staged_signs ||
+                   og.awq != staged_awq) {
+            stage_x<BF16>(p, xin, og.signs, og.awq, lds, k0, kc, gm.tid, gm.nthreads);
+            staged = true;
+            staged_x = xin;
+            staged_signs = og.signs;
+            staged_awq = og.awq;
+        }
+        FLUTE_TRACE(2);
+        float acc[8];
+#pragma unroll
+        for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
+        for (int si = 0; si < og.nstreams; ++si) {
+            const GemvStream st = kp->seg[so == 1 ? 1 : si0].st[si];
+            if (BFIX != 0 && so == 0 && si == 0) {
+                if constexpr (BFIX != 0) {
+                    stream_tables<BF>(st, gm, lds, first);
+                    __syncthreads();
+                    FLUTE_TRACE(3);
+                    stream_loop<BF, BF16>(p, og, st, gm, lds, first, acc);
+                    __syncthreads();
+                    FLUTE_TRACE(4);
+                }
+            } else {
+                run_stream_any<BF16, BFIX>(p, og, st, gm, lds, acc);
+            }
+        }
+
+        // fold the lanes that share rows: 16 (i, kt) lanes, then the tiles of a load
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
-            const int row = (u >> 1) * 64 + (a >> 1) * 16 + (a & 1) * 8 + 4 * (u & 1) + (L >> 4);
-            red[row] = acc[a];
+            float v = row16_sum(acc[a]);
+            if (p.lpg_log2 <= 5) v += __shfl_xor(v, 32);
+            if (p.lpg_log2 == 4) v += __shfl_xor(v, 16);
+            acc[a] = v;
+        }
+        if (gm.L < lpg && (gm.L & 15) == 0) {
+#pragma unroll
+            for (int a = 0; a < 8; ++a)
+                red[(so * gm.nwaves + gm.w) * 32 + (gm.L >> 4) * 8 + a] = acc[a];
         }
     }
     __syncthreads();
 
-    // ---- publish, take a ticket, let the last arrival finish the tile ---------
-    int *flag = (int *)(lds + p.lds_xb + kGemvMaxRank * 4);
-    if (!direct) {
-        if (tid < 128)
-            p.P[(size_t)(jb.slot0 + s) * p.p_stride + sg.n0 + t * 128 + tid] = red[tid];
-        __threadfence();
+    // ---- one thread per owned row: fold the wavefronts in fixed order ----------
+    const bool owner = gm.tid < rw;
+    const int cg_o = gm.cg0 + (gm.tid >> 3);
+    const int n = gm.t * 128 + row_of(cg_o, gm.tid & 7);
+    float yv[2] = {0.0f, 0.0f};
+    if (owner) {
+#pragma unroll
+        for (int so = 0; so < 2; ++so) {
+            if (so >= nout) break;
+            float y = 0.0f;
+            for (int w = 0; w < gm.nwaves; ++w) y += red[(so * gm.nwaves + w) * 32 + gm.tid];
+            yv[so] = y;
+        }
+    }
+
+    if (p.split > 1) {
+        // publish the partials of this K range, take a ticket, let the last
+        // arrival finish the rows
+        int *flag = (int *)(red + 2 * gm.nwaves * 32);
+        if (owner) {
+#pragma unroll
+            for (int so = 0; so < 2; ++so) {
+                if (so >= nout) break;
+                const int og_n0 = kp->seg[so == 1 ? 1 : si0].n0;
+                ws_store(p.P + (size_t)s * p.p_stride + og_n0 + n, yv[so]);
+            }
+        }
+        // the stores are acknowledged by the device-coherent level before the ticket
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
-        if (tid == 0) {
-            const int old = atomicAdd(p.tickets + sg.ticket0 + t, 1);
-            *flag = (old == sg.arrivals - 1);
+        if (gm.tid == 0) {
+            const int old = __hip_atomic_fetch_add(p.tickets + sg.ticket0 + sl, 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+            *flag = (old == p.split - 1);
         }
         __syncthreads();
         if (!*flag) return;
-        __threadfence();
+        if (owner) {
+#pragma unroll
+            for (int so = 0; so < 2; ++so) {
+                if (so >= nout) break;
+                const float *col = p.P + kp->seg[so == 1 ? 1 : si0].n0 + n;
+                float y = 0.0f;
+                for (int sb = 0; sb < p.split; sb += 8) {     // 8 independent loads in flight
+                    float part[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        part[j] = (sb + j < p.split) ? ws_load(col + (size_t)(sb + j) * p.p_stride)
+                                                     : 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) y += part[j];
+                }
+                yv[so] = y;
+            }
+        }
+        if (gm.tid == 0)
+            __hip_atomic_store(p.tickets + sg.ticket0 + sl, 0, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    // residual coefficients x . resB[r], folded over the splits in fixed order
-    const int nseg_out = p.silu_mul ? 2 : 1;
-    float yv[2] = {0.0f, 0.0f};
+    if (owner) {
 #pragma unroll
-    for (int so = 0; so < 2; ++so) {
-        if (so >= nseg_out) break;                 // uniform
-        const GemvSeg &og = p.silu_mul ? (so == 0 ? p.seg[0] : p.seg[1]) : sg;
-        if (og.R > 0 && !direct) {
-            __syncthreads();
-            for (int r = tid; r < og.R; r += kGemvThreads) {
-                float c = 0.0f;
-                for (int sp = 0; sp < p.split; ++sp)
-                    c += __hip_atomic_load(p.P + (size_t)sp * p.p_stride + og.r0 + r,
-                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                xB[r] = c;
-            }
-            __syncthreads();
-        }
-        if (tid < 128) {
-            const int n = t * 128 + tid;
-            float y = fold_row(p, og, n, !direct, red[tid]);
+        for (int so = 0; so < 2; ++so) {
+            if (so >= nout) break;
+            const GemvSeg og = kp->seg[so == 1 ? 1 : si0];
+            float y = yv[so];
             if (og.R > 0) {
                 const uint16_t *ra = og.resA + (size_t)n * og.R;
                 for (int r = 0; r < og.R; ++r)
-                    y = fmaf(xB[r], p.act_bf16 ? bf2f(ra[r]) : h2f(ra[r]), y);
+                    y = fmaf(og.xb[r], p.act_bf16 ? bf2f(ra[r]) : h2f(ra[r]), y);
             }
             if (og.bias) y += p.act_bf16 ? bf2f(og.bias[n]) : h2f(og.bias[n]);
             yv[so] = y;
         }
-    }
-    if (tid < 128) {
-        const int n = t * 128 + tid;
         float y = yv[0];
-        uint16_t *out = sg.out;
-        if (p.silu_mul) {
-            y = (yv[0] / (1.0f + expf(-yv[0]))) * yv[1];
-            out = p.seg[0].out;
-        }
-        out[n] = round_act(y, p.act_bf16);
+        if (p.silu_mul) y = (yv[0] / (1.0f + expf(-yv[0]))) * yv[1];
+        sg.out[n] = round_act(y, p.act_bf16);
     }
-    if (!direct && tid == 0) {
-        __hip_atomic_store(p.tickets + sg.ticket0 + t, 0, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-    }
+    FLUTE_TRACE(5);
 }
 
-template <bool BF16>
-__global__ void __launch_bounds__(kGemvThreads) gemv_kernel(const GemvParams p) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    // Pick this workgroup's job and weight with static indices only, so that the
-    // kernel arguments stay in scalar registers.
-    GemvJob jb = p.job[0];
-#pragma unroll
-    for (int j = 1; j < kGemvMaxJobs; ++j)
-        if (j < p.njobs && (int)blockIdx.x >= p.job[j].tile0) jb = p.job[j];
-    GemvSeg sg = p.seg[0];
-#pragma unroll
-    for (int i = 1; i < kGemvMaxSegs; ++i)
-        if (jb.seg == i) sg = p.seg[i];
-    switch (jb.bits) {
-        case 4: gemv_body<4, BF16>(p, jb, sg, lds); break;
-        case 3: gemv_body<3, BF16>(p, jb, sg, lds); break;
-        case 2: gemv_body<2, BF16>(p, jb, sg, lds); break;
-        default: gemv_body<1, BF16>(p, jb, sg, lds); break;
+// Residual coefficients: xb[r] = sum_k x[k] * resB[r][k] in fp32, one workgroup
+// per residual row, x taken as given (already rotated).  A thread-strided sum
+// followed by a fixed-order tree: deterministic.
+__global__ void __launch_bounds__(256) residual_coeff_kernel(const uint16_t *x,
+                                                             const uint16_t *resB, float *xb,
+                                                             int K, int act_bf16) {
+    __shared__ float part[256];
+    const uint16_t *row = resB + (size_t)blockIdx.x * K;
+    float s = 0.0f;
+    for (int k = threadIdx.x; k < K; k += 256) {
+        const float a = act_bf16 ? bf2f(x[k]) : h2f(x[k]);
+        const float b = act_bf16 ? bf2f(row[k]) : h2f(row[k]);
+        s = fmaf(a, b, s);
     }
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int step = 128; step > 0; step >>= 1) {
+        if ((int)threadIdx.x < step) part[threadIdx.x] += part[threadIdx.x + step];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) xb[blockIdx.x] = part[0];
 }
 
 }  // namespace flute
