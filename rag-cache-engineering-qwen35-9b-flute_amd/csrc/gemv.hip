@@ -1,6 +1,7 @@
 // Launchers of the M = 1 LUT GEMV family: single weight, merged gate/up with
 // SiLU*mul, several weights sharing one input, and the two-launch MLP block.
 #include "gemv_kernel.h"
+#include "gemv4_kernel.h"
 #include "host_common.h"
 
 #include <cmath>
@@ -80,8 +81,10 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
     *split = sp;
     int wv = env_int("FLUTE_GEMV_WAVES", 0);
     if (wv != 1 && wv != 2 && wv != 4 && wv != 8) {
+        // four wavefronts with eight loads each in flight measured best; eight when a
+        // workgroup has a long K range to itself
         const int units = (G / sp) / (32 / best_rw);
-        wv = units >= 16 ? 8 : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
+        wv = units >= 64 ? 8 : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
     }
     *waves = wv;
 }
@@ -141,9 +144,21 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     size_t xb_off = 0, xrot_off = 0;
     int n0 = 0, col = 0, ticket = 0;
     size_t tab_bytes = 0;
-    // LDS: tables/scratch | x slice | row sums.  Two workgroups per CU when possible.
+    // LDS: tables/scratch | x slice | row sums.  The table stride is the largest
+    // that still lets the whole grid be resident at once (one round of
+    // workgroups), since a second round repeats the start-up latency.
     int budget = env_int("FLUTE_GEMV_TABLE_LOG2", 0);
-    if (budget < 12 || budget > 17) budget = (kc * 2 + 4096 + 65536 <= kLdsPerCU / 2) ? 16 : 15;
+    if (budget < 12 || budget > 17) {
+        long wgs = 0;
+        for (int i = 0; i < (silu_mul ? 1 : count); ++i) wgs += (long)(segs[i].N / rw) * split;
+        long per_cu = (wgs + kNumCU - 1) / kNumCU;
+        if (per_cu > 4) per_cu = 4;
+        if (per_cu < 1) per_cu = 1;
+        const long fixed = kc * 2 + 4096;
+        budget = 14;
+        for (int cand = 16; cand >= 14; --cand)
+            if (((1L << cand) + fixed) * per_cu <= kLdsPerCU) { budget = cand; break; }
+    }
     for (int i = 0; i < count; ++i) {
         const flute_linear &w = segs[i];
         GemvSeg &sg = p.seg[i];
@@ -265,13 +280,65 @@ flute_status launch_typed(Plan &plan, hipStream_t stream) {
     return FLUTE_OK;
 }
 
+template <int LPGL, int NW, int ES, bool BF16, bool MULTI>
+flute_status launch_fast4m(Plan &plan, hipStream_t stream) {
+    static bool attr_done = false;
+    if (!attr_done) {
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv4_kernel<LPGL, NW, ES, BF16, MULTI>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            (int)kLdsPerCU));
+        attr_done = true;
+    }
+#ifdef FLUTE_GEMV_TRACE
+    {
+        const char *e = std::getenv("FLUTE_GEMV_TRACE_PTR");
+        plan.p.trace = e ? (unsigned long long *)std::strtoull(e, nullptr, 0) : nullptr;
+    }
+#endif
+    dim3 grid(plan.grid_x, plan.p.split);
+    hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, ES, BF16, MULTI>), grid, dim3(NW * 64),
+                       plan.lds_bytes, stream, plan.p);
+    FLUTE_HIP_CHECK(hipGetLastError());
+    return FLUTE_OK;
+}
+
+template <int LPGL, int NW, int ES, bool BF16>
+flute_status launch_fast4(Plan &plan, hipStream_t stream) {
+    const bool multi = plan.p.nsegs > 1 && !plan.p.silu_mul;
+    return multi ? launch_fast4m<LPGL, NW, ES, BF16, true>(plan, stream)
+                 : launch_fast4m<LPGL, NW, ES, BF16, false>(plan, stream);
+}
+
+template <int LPGL, bool BF16>
+flute_status launch_fast4_shape(Plan &plan, int nw, int es, hipStream_t stream) {
+    if (nw == 4) return es == 8 ? launch_fast4<LPGL, 4, 8, BF16>(plan, stream)
+                                : launch_fast4<LPGL, 4, 7, BF16>(plan, stream);
+    return es == 8 ? launch_fast4<LPGL, 8, 8, BF16>(plan, stream)
+                   : launch_fast4<LPGL, 8, 7, BF16>(plan, stream);
+}
+
 template <bool BF16>
 flute_status launch_width(Plan &plan, hipStream_t stream) {
     // one width for the whole launch -> the instantiation specialised for it
     int bits = plan.p.seg[0].st[0].bits;
-    for (int i = 0; i < plan.p.nsegs; ++i)
-        for (int st = 0; st < plan.p.seg[i].nstreams; ++st)
+    int es = plan.p.seg[0].st[0].es;
+    bool one_group = true;
+    for (int i = 0; i < plan.p.nsegs; ++i) {
+        one_group &= plan.p.seg[i].gs >= 128;
+        for (int st = 0; st < plan.p.seg[i].nstreams; ++st) {
             if (plan.p.seg[i].st[st].bits != bits) bits = 0;
+            if (plan.p.seg[i].st[st].es != es) es = 0;
+        }
+    }
+    const int nw = plan.threads / 64;
+    if (bits == 4 && one_group && (es == 7 || es == 8) && (nw == 4 || nw == 8) &&
+        env_int("FLUTE_GEMV_NO_FAST", 0) == 0) {
+        switch (plan.p.lpg_log2) {
+            case 4: return launch_fast4_shape<4, BF16>(plan, nw, es, stream);
+            case 5: return launch_fast4_shape<5, BF16>(plan, nw, es, stream);
+            default: return launch_fast4_shape<6, BF16>(plan, nw, es, stream);
+        }
+    }
     switch (bits) {
         case 4: return launch_typed<BF16, 4>(plan, stream);
         case 3: return launch_typed<BF16, 3>(plan, stream);

@@ -13,7 +13,9 @@ namespace flute {
 // LPGL = log2(lanes per 64-k tile) = log2(2 * rows per workgroup): 4, 5, 6.
 // NW   = wavefronts per workgroup.
 // ES   = log2(table stride): 8 (v_perm addressing, 64 KB) or 7 (32 KB).
-template <int LPGL, int NW, int ES, bool BF16>
+// MULTI = several independent weights share the launch (the descriptor is then
+//         picked by grid column, which costs a dependent scalar load).
+template <int LPGL, int NW, int ES, bool BF16, bool MULTI>
 __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int NT = NW * 64;
@@ -21,7 +23,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
     constexpr int GPI = 64 >> LPGL;                 // 64-k tiles per wavefront load
     constexpr int RW = LPG >> 1;                    // rows per workgroup
     constexpr int SPT = 128 / RW;                   // row slices per tile
-    constexpr int PF = 4;                           // wavefront loads in flight per lane
+    constexpr int PF = NW == 4 ? 8 : 4;             // wavefront loads in flight per lane
     constexpr int XV = 2;                           // 16-byte activation loads per thread
     constexpr int STRIDE = 1 << ES;                 // table bytes per entry
     constexpr int CHUNKS = STRIDE / 16;             // 16-byte pieces of one entry's replicas
@@ -31,7 +33,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     int si0 = 0;
-    if (!p.silu_mul) {
+    if (MULTI && !p.silu_mul) {
 #pragma unroll
         for (int i = 1; i < kGemvMaxSegs; ++i)
             if (i < p.nsegs && (int)blockIdx.x >= p.seg[i].col0) si0 = i;
@@ -62,7 +64,12 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
                            (uint32_t)w * unit_bytes;
     constexpr uint32_t step = NW * GPI * 4096u;
     const int xi = gsub * 32 + (l & 3) * 8 + ((l >> 2) & 3) + w * (GPI * 32);
-    const uint32_t slot = ES == 8 ? (uint32_t)L * 4u : (uint32_t)(L & 31) * 4u;
+    // Lookup addresses are formed as absolute LDS addresses, so the (zero) base of
+    // the dynamic LDS block is folded into the per-lane replica offset once
+    // instead of being added after every v_perm.
+    typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    const uint32_t slot = lds_base + (ES == 8 ? (uint32_t)L * 4u : (uint32_t)(L & 31) * 4u);
     const int e_own = tid & 255;                    // table entry this thread writes
     const int share = tid >> 8;
 
@@ -71,6 +78,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
     const float *staged_signs = nullptr, *staged_awq = nullptr;
     bool staged = false;
 
+    FLUTE_TRACE(0);
     for (int so = 0; so < nout; ++so) {
         const int si_seg = so == 1 ? 1 : si0;
         const uint16_t *xin = kp->seg[si_seg].xsrc ? kp->seg[si_seg].xsrc : p.x;
@@ -107,6 +115,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
                 if (n < my_units) q[n] = *(const uint4 *)(qrow + (lane0 + (uint32_t)n * step));
             }
 
+            FLUTE_TRACE(1);
             // ---- activations into LDS ---------------------------------------------
             if (si == 0 && restage) {
                 if (x_direct) {
@@ -139,6 +148,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
                     *(uint4 *)(ent + (((k + tid) & (CPT - 1)) << 4)) = v4;
             }
             __syncthreads();
+            FLUTE_TRACE(2);
 
             // ---- K loop -----------------------------------------------------------
             for (int nb = 0; nb < my_units; nb += PF) {
@@ -159,11 +169,11 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
                                 uint32_t addr;
                                 if constexpr (ES == 8) {
                                     addr = __builtin_amdgcn_perm(wq[v], slot,
-                                                                 0x0c0c0000u | ((4u + j) << 8));
+                                                                 0x03020000u | ((4u + j) << 8));
                                 } else {
-                                    addr = (((wq[v] >> (8 * j)) & 0xffu) << ES) | slot;
+                                    addr = (((wq[v] >> (8 * j)) & 0xffu) << ES) + slot;
                                 }
-                                const uint32_t e = *(const uint32_t *)(lds + addr);
+                                const uint32_t e = *(LdsWord)addr;
                                 acc[v * 2 + (j >> 1)] =
                                     dot2<BF16>(e, (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
                             }
@@ -171,6 +181,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
                     }
                 }
             }
+            FLUTE_TRACE(3);
             __syncthreads();                       // the table region is rewritten next
         }
 
@@ -188,6 +199,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
         }
     }
     __syncthreads();
+    FLUTE_TRACE(4);
 
     // ---- one thread per owned row --------------------------------------------------
     if (tid >= RW && p.split == 1) return;
@@ -264,6 +276,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
         if (p.silu_mul) y = (yv[0] / (1.0f + expf(-yv[0]))) * yv[1];
         kp->seg[si0].out[n] = round_act(y, p.act_bf16);
     }
+    FLUTE_TRACE(5);
 }
 
 }  // namespace flute

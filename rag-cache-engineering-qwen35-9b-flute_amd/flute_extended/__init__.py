@@ -317,7 +317,8 @@ def gemv_multi_supported(K: int, tiles_total: int, specs, residual_rank_total: i
     return all(_lds_ok(128, K, b1, b2, gs, fht) for b1, b2, gs in specs)
 
 
-def qgemm_gemv_multi(A: torch.Tensor, seg_table: torch.Tensor) -> None:
+def qgemm_gemv_multi(A: torch.Tensor, seg_table: torch.Tensor,
+                     lut_dtype: Optional[torch.dtype] = None) -> None:
     """2-4 weights sharing one input row in one launch.  seg_table: CPU int64
     [count, 15] of raw data_ptr() values, columns
     [q1, lut1, q2, lut2, resB, resA, bias, C, N, R, b1, b2, gs, signs, s]."""
@@ -327,7 +328,7 @@ def qgemm_gemv_multi(A: torch.Tensor, seg_table: torch.Tensor) -> None:
     if not (seg_table.device.type == "cpu" and seg_table.dtype == torch.int64
             and seg_table.dim() == 2 and seg_table.size(1) == 15):
         raise ValueError("qgemm_gemv_multi: seg_table must be a CPU int64 [count, 15] tensor")
-    _qgemm_gemv_multi(A, seg_table)
+    _qgemm_gemv_multi(A, seg_table, lut_dtype)
 
 
 def gemv_mlp_available() -> bool:
@@ -347,8 +348,10 @@ def gemv_mlp_supported(K: int, N: int, specs, residual_rank_g: int = 0, residual
     return all(_lds_ok(N, K, b1, b2, gs, fht) for b1, b2, gs in specs)
 
 
-def qgemm_gemv_mlp(A: torch.Tensor, seg_table: torch.Tensor, C: torch.Tensor) -> torch.Tensor:
-    """C = silu(gate(A)) * up(A) in one launch; seg_table row 0 = gate, row 1 = up."""
+def qgemm_gemv_mlp(A: torch.Tensor, seg_table: torch.Tensor, C: torch.Tensor,
+                   lut_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """C = silu(gate(A)) * up(A) in one launch; seg_table row 0 = gate, row 1 = up.
+    The table holds raw pointers: LUTs are float16 unless lut_dtype says bfloat16."""
     if not (A.dim() == 2 and A.shape[0] == 1 and A.is_contiguous()
             and A.dtype in (torch.float16, torch.bfloat16)):
         raise ValueError("qgemm_gemv_mlp: A must be a contiguous [1, K] float16/bfloat16 tensor")
@@ -357,7 +360,7 @@ def qgemm_gemv_mlp(A: torch.Tensor, seg_table: torch.Tensor, C: torch.Tensor) ->
         raise ValueError("qgemm_gemv_mlp: seg_table must be a CPU int64 [2, 15] tensor")
     if not (C.dtype == A.dtype and C.is_contiguous()):
         raise ValueError("qgemm_gemv_mlp: C must be a contiguous output buffer of A's dtype")
-    return _qgemm_gemv_mlp(A, seg_table, C)
+    return _qgemm_gemv_mlp(A, seg_table, C, lut_dtype)
 
 
 __all__ = [

@@ -1,0 +1,177 @@
+"""GPU parity of the M = 1 LUT GEMV family against the oracle, through the
+flute_extended op surface (which calls the C ABI).
+
+Tolerance (stated by the benchmark contract): relative L2 <= 1e-3 against the
+reference arithmetic for fp32 accumulate with a 16-bit output.  The oracle value
+is the fp64 closed form rounded once to the output dtype, i.e. what an exact
+fp32-accumulate kernel would produce; the upstream torch path
+(oracle.linear_reference) is compared as well where it rounds at the same point.
+Index decoding is additionally checked bit-exactly: a one-hot input must return
+the dequantised column.
+"""
+import pytest
+import torch
+
+import flute_extended as fx
+import flute_oracle as O
+from _util import make_weight, make_x, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-3
+
+
+def _run(w, x, entry=None, signs=None, awq=None, **extra):
+    entry = entry or fx.qgemm_gemv_splitk_stream
+    return entry(x.to(DEV), w["blob_d"], w["lut_d"], w["bits"], w["gs"],
+                 indices2=w.get("blob2_d"), lut2=w.get("lut2_d"), bitwidth2=w["bits2"],
+                 resB=w.get("resB_d"), resA=w.get("resA_d"), bias=w.get("bias_d"),
+                 rot_signs=None if signs is None else signs.to(DEV),
+                 awq_scale=None if awq is None else awq.to(DEV), **extra)
+
+
+def _exact(w, x):
+    return O.linear_exact(x, w["blob"].numpy(), w["lut"], w["N"], w["K"], w["gs"], w["bits"],
+                          w["blob2"].numpy() if w["bits2"] else None, w["lut2"], w["bits2"],
+                          w["resA"], w["resB"], w["bias"])
+
+
+CASES = [
+    # N, K, bits, gs, bits2, rank, bias
+    (128, 64, 4, 128, 0, 0, False),
+    (256, 512, 4, 128, 0, 0, False),
+    (1024, 4096, 4, 128, 0, 0, False),
+    (1024, 4096, 4, 64, 0, 0, False),
+    (1024, 2048, 4, 32, 0, 0, False),
+    (1024, 2048, 4, 16, 0, 0, False),
+    (1024, 2048, 4, 512, 0, 0, False),
+    (384, 1024, 4, 256, 0, 0, False),       # N not a multiple of the group size
+    (512, 1024, 3, 128, 0, 0, False),
+    (512, 1024, 2, 128, 0, 0, False),
+    (512, 1024, 1, 128, 0, 0, False),
+    (512, 1024, 3, 32, 0, 0, False),
+    (512, 1024, 2, 16, 0, 0, False),
+    (512, 1024, 1, 64, 0, 0, False),
+    (512, 1024, 4, 128, 1, 0, False),
+    (512, 1024, 1, 128, 4, 0, True),
+    (512, 1024, 3, 128, 3, 16, True),
+    (512, 1024, 2, 64, 3, 0, False),
+    (512, 1024, 4, 128, 4, 4, False),
+    (512, 2048, 4, 128, 0, 64, True),
+    (256, 1024, 4, 128, 0, 256, False),
+]
+
+
+@pytest.mark.parametrize("N,K,bits,gs,bits2,rank,bias", CASES)
+def test_gemv_fp16(N, K, bits, gs, bits2, rank, bias):
+    w = make_weight(N, K, bits, gs, seed=N + K + bits, bits2=bits2, rank=rank, bias=bias,
+                    device=DEV)
+    x = make_x(1, K, seed=7)
+    y = _run(w, x).cpu()
+    assert y.shape == (1, N) and y.dtype == torch.float16
+    assert rel_l2(y, _exact(w, x).half()) <= TOL
+    assert torch.equal(y, _run(w, x).cpu())            # deterministic
+
+
+@pytest.mark.parametrize("split", [1, 2, 4, 8, 16])
+def test_forced_splits_agree(split):
+    w = make_weight(512, 4096, 4, 128, seed=3, rank=8, bias=True, device=DEV)
+    x = make_x(1, 4096, seed=5)
+    y = _run(w, x, split=split).cpu()
+    assert rel_l2(y, _exact(w, x).half()) <= TOL
+    assert torch.equal(y, _run(w, x, split=split).cpu())
+
+
+def test_plain_entry_and_contract():
+    w = make_weight(512, 1024, 4, 128, seed=9, rank=16, bias=True, device=DEV)
+    x = make_x(1, 1024, seed=2)
+    y = _run(w, x, entry=fx.qgemm_gemv_stream).cpu()
+    assert rel_l2(y, _exact(w, x).half()) <= TOL
+    w2 = make_weight(512, 1024, 4, 128, seed=9, rank=32, device=DEV)
+    with pytest.raises(RuntimeError):
+        _run(w2, x, entry=fx.qgemm_gemv_stream)        # rank cap of the plain entry
+    with pytest.raises(RuntimeError):
+        fx.qgemm_gemv_splitk_stream(make_x(2, 1024).to(DEV), w["blob_d"], w["lut_d"], 4, 128)
+
+
+@pytest.mark.parametrize("lut_dtype", [torch.float16, torch.bfloat16])
+def test_gemv_bf16_activations(lut_dtype):
+    N, K = 512, 4096
+    w = make_weight(N, K, 4, 128, seed=4, lut_dtype=lut_dtype, act_dtype=torch.bfloat16,
+                    bias=True, rank=4, device=DEV)
+    x = make_x(1, K, seed=6, dtype=torch.bfloat16)
+    y = _run(w, x).cpu()
+    assert y.dtype == torch.bfloat16
+    assert rel_l2(y, _exact(w, x).bfloat16()) <= TOL
+    # the upstream torch path on the same inputs, no residual/bias: same rounding point
+    w0 = make_weight(N, K, 4, 128, seed=4, lut_dtype=lut_dtype, act_dtype=torch.bfloat16,
+                     device=DEV)
+    ref = O.linear_reference(x, w0["blob"].numpy(), w0["lut"], N, K, 128, 4)
+    assert rel_l2(_run(w0, x).cpu(), ref) <= TOL
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 128), (3, 64), (2, 128), (1, 32), (4, 16)])
+def test_one_hot_input_returns_the_dequantised_column(bits, gs):
+    """y = W[:, k] exactly when x = e_k: checks every lookup of the K loop."""
+    N, K = 512, 512
+    w = make_weight(N, K, bits, gs, seed=bits * 7 + gs, device=DEV)
+    W = O.dequant(w["blob"], w["lut"], N, K, gs, bits)
+    for k in (0, 1, 9, 63, 64, 200, 511):
+        x = torch.zeros(1, K, dtype=torch.float16); x[0, k] = 1.0
+        assert torch.equal(_run(w, x).cpu()[0].float(), W[:, k])
+
+
+def test_one_hot_at_benchmark_size():
+    N, K = 12288, 4096
+    w = make_weight(N, K, 4, 128, seed=1, device=DEV)
+    idx, lut = w["idx"].long(), w["lut"].float()
+    rows = torch.arange(N) // 128
+    for k in (0, 1337, 4095):
+        x = torch.zeros(1, K, dtype=torch.float16); x[0, k] = 1.0
+        assert torch.equal(_run(w, x).cpu()[0].float(), lut[rows, idx[:, k]])
+
+
+@pytest.mark.parametrize("N,K", [(12288, 4096), (4096, 12288), (1024, 4096), (512, 4096)])
+def test_benchmark_shapes(N, K):
+    w = make_weight(N, K, 4, 128, seed=N % 97, device=DEV)
+    x = make_x(1, K, seed=3)
+    y = _run(w, x).cpu()
+    assert rel_l2(y, _exact(w, x).half()) <= TOL
+    # linearity, a size-independent property: f(2x) == 2 f(x) bit for bit wherever the
+    # fp16 output is a normal number (doubling is exact in fp32 and commutes with the
+    # final rounding; subnormal outputs have a fixed quantum, so they are excluded)
+    normal = y.abs() >= 2.0 ** -13
+    assert normal.float().mean() > 0.99
+    assert torch.equal(_run(w, x * 2).cpu()[normal], (y * 2)[normal])
+
+
+@pytest.mark.parametrize("K,awq,dtype", [(4096, False, torch.float16), (12288, True, torch.float16),
+                                         (1536, False, torch.float16), (4096, True, torch.bfloat16)])
+def test_fused_rotation_is_bit_identical_to_rotate_then_gemv(K, awq, dtype):
+    import fht
+    N = 512
+    w = make_weight(N, K, 4, 128, seed=5, rank=8, bias=True, act_dtype=dtype, device=DEV)
+    x = make_x(1, K, seed=8, dtype=dtype)
+    signs = O.rotation_signs(K, 21)
+    s = (torch.rand(K, generator=torch.Generator().manual_seed(1)) + 0.5) if awq else None
+    fused = _run(w, x, signs=signs, awq=s)
+    xr = fht.fht_apply_awq(x.to(DEV), signs.to(DEV), s.to(DEV), backend="kernel") if awq \
+        else fht.fht_apply(x.to(DEV), signs.to(DEV), backend="kernel")
+    chain = _run(w, xr.cpu())
+    assert torch.equal(fused, chain)
+    w0 = make_weight(N, K, 4, 128, seed=5, act_dtype=dtype, device=DEV)   # fused prologue path
+    assert torch.equal(_run(w0, x, signs=signs, awq=s), _run(w0, xr.cpu()))
+    xo = O.fht_awq_reference(x, signs, s) if awq else O.fht_reference(x, signs)
+    assert rel_l2(fused.cpu(), _exact(w, xo).to(dtype)) <= (TOL if dtype == torch.float16 else 4e-3)
+
+
+def test_block_rotation_mode():
+    """Equal 128-column rotation blocks (the benchmark's wording), defined by the
+    closed form oracle.block_fht_reference."""
+    N, K = 512, 4096
+    w = make_weight(N, K, 4, 128, seed=6, device=DEV)
+    x = make_x(1, K, seed=9)
+    signs = torch.ones(K)
+    y = _run(w, x, signs=signs, rot_block=128).cpu()
+    xo = O.block_fht_reference(x, 128, signs)
+    assert rel_l2(y, _exact(w, xo).half()) <= TOL

@@ -1,0 +1,270 @@
+"""Host-side contract, no GPU needed: the C ABI library loads and exports every
+symbol include/flute_hip.h declares; every refusal upstream lists
+(test_flute.py:226-262, src/kernel_gemv.cu:338-454) raises the same exception
+type here; the gate mirrors and the module layer behave as documented."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import flute_extended as fx
+from flute_extended import _C, _lib
+import palettized_modules as pm
+import fht
+import flute_oracle as O
+from _util import make_weight, make_x
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "flute_hip.h")).read()
+    body = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(flute_[a-z0-9_]+)\s*\(", body))
+    assert declared == set(_lib.SYMBOLS), declared ^ set(_lib.SYMBOLS)
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.flute_abi_version() == 1
+    assert _lib.lib.flute_target_arch() == b"gfx950"
+
+
+def test_struct_layout_matches_header():
+    # 9 pointers, 2 int64, 9 int32 -> 8*9 + 16 + 36 = 124, padded to 128
+    assert ctypes.sizeof(_lib.FluteLinear) == 128
+    assert _lib.FluteLinear.q1_bytes.offset == 72 and _lib.FluteLinear.lut_rows.offset == 88
+
+
+def _desc(N=256, K=128, b1=4, b2=0, gs=128, R=0, **over):
+    w = _lib.FluteLinear()
+    w.q1 = w.lut1 = 4096
+    if b2:
+        w.q2 = w.lut2 = 4096
+    if R:
+        w.resA = w.resB = 4096
+    w.N, w.K, w.R, w.b1, w.b2, w.group_size = N, K, R, b1, b2, gs
+    w.q1_bytes, w.q2_bytes = N * K * b1 // 8, N * K * b2 // 8
+    w.lut_rows = (N + gs - 1) // gs
+    w.lut_dtype = _lib.F16
+    for k, v in over.items():
+        setattr(w, k, v)
+    return w
+
+
+@pytest.mark.parametrize("over,code", [
+    ({}, _lib.FLUTE_OK),
+    ({"b1": 5}, _lib.FLUTE_ERR_INVALID),
+    ({"b2": 7}, _lib.FLUTE_ERR_INVALID),
+    ({"K": 96}, _lib.FLUTE_ERR_INVALID),
+    ({"N": 200}, _lib.FLUTE_ERR_INVALID),
+    ({"group_size": 48}, _lib.FLUTE_ERR_INVALID),
+    ({"group_size": 8}, _lib.FLUTE_ERR_INVALID),
+    ({"q1_bytes": 100}, _lib.FLUTE_ERR_INVALID),          # truncated blob
+    ({"lut_rows": 7}, _lib.FLUTE_ERR_INVALID),            # wrong LUT geometry
+    ({"q1": 4097}, _lib.FLUTE_ERR_INVALID),               # misaligned indices
+    ({"q1": None}, _lib.FLUTE_ERR_INVALID),
+    ({"R": 300, "resA": 4096, "resB": 4096}, _lib.FLUTE_ERR_INVALID),
+    ({"resA": 4096}, _lib.FLUTE_ERR_INVALID),             # resA without resB
+    ({"awq": 4096}, _lib.FLUTE_ERR_INVALID),              # awq without signs
+    ({"lut_dtype": 2}, _lib.FLUTE_ERR_INVALID),
+])
+def test_c_validation(over, code):
+    w = _desc(**over)
+    assert _lib.lib.flute_validate(ctypes.byref(w), 0) == code
+    if code != _lib.FLUTE_OK:
+        assert _lib.last_error()
+
+
+def test_c_entry_points_refuse_before_touching_the_device():
+    w = _desc()
+    assert _lib.lib.flute_gemv(ctypes.byref(w), None, 4096, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_gemv(ctypes.byref(w), 4096, 4096, 7, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_gemv(ctypes.byref(w), 4096, 4096, 0, 3, None) == _lib.FLUTE_ERR_INVALID  # split !| K/64
+    w2 = _desc(lut_dtype=_lib.BF16)
+    assert _lib.lib.flute_gemv(ctypes.byref(w2), 4096, 4096, _lib.F16, 0, None) \
+        == _lib.FLUTE_ERR_UNSUPPORTED
+    assert _lib.lib.flute_fht(4096, 4096, None, 4096, 1, 100, 0, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_fht(4096, 4096, 4096, 4096, 1, 128, 0, 1, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_fht(4096, 4096, None, 4096, 1, 32768, 0, 0, 0, None) \
+        == _lib.FLUTE_ERR_UNSUPPORTED
+    g, u = _desc(), _desc(N=384)
+    assert _lib.lib.flute_gemv_mlp(ctypes.byref(g), ctypes.byref(u), 4096, 4096, 0, 0, None) \
+        == _lib.FLUTE_ERR_INVALID
+
+
+def _cpu_args(N=256, K=128, b=4, gs=128, dtype=torch.float16):
+    w = make_weight(N, K, b, gs, seed=1, act_dtype=dtype)
+    return make_x(1, K, dtype=dtype), w
+
+
+def test_tensor_level_refusals_raise_runtimeerror():
+    x, w = _cpu_args()
+    call = lambda **kw: fx.qgemm_gemv_splitk_stream(
+        kw.pop("A", x), kw.pop("indices", w["blob"]), kw.pop("lut", w["lut"]),
+        kw.pop("bitwidth", 4), kw.pop("group_size", 128), **kw)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        call()                                                     # valid shapes, CPU tensors
+    with pytest.raises(RuntimeError, match="M == 1"):
+        call(A=make_x(2, 128))
+    with pytest.raises(RuntimeError, match="byte count"):
+        call(indices=w["blob"][:-7])                                # truncated blob
+    with pytest.raises(RuntimeError, match="lut must be"):
+        call(lut=w["lut"][:, :8].contiguous())                      # wrong LUT width
+    with pytest.raises(RuntimeError, match="group_size"):
+        call(group_size=48)
+    with pytest.raises(RuntimeError, match="bitwidth"):
+        call(bitwidth=5)
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        call(A=make_x(1, 96))
+    with pytest.raises(RuntimeError, match="float16"):
+        call(A=make_x(1, 128, dtype=torch.float32))
+    with pytest.raises(RuntimeError, match="together"):
+        call(resB=torch.zeros(4, 128, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="rank"):
+        call(resB=torch.zeros(300, 128, dtype=torch.float16),
+             resA=torch.zeros(256, 300, dtype=torch.float16))
+    with pytest.raises(ValueError, match="awq_scale"):
+        call(awq_scale=torch.ones(128))                             # awq without signs
+    with pytest.raises(ValueError, match="rot_signs"):
+        call(rot_signs=torch.ones(64))
+    with pytest.raises(RuntimeError, match="group_size"):
+        fx.qgemm_gemv_stream(x, w["blob"], w["lut"], 4, 32)         # plain entry: gs >= 64 only
+
+
+def test_layout_string_guards():
+    x, w = _cpu_args()
+    with pytest.raises(ValueError):
+        fx.qgemm_per_group_lut(x, w["blob"], w["lut"], 4, 128, indices_layout="idx9")
+    with pytest.raises(ValueError):
+        fx.qgemm_per_group_lut(x, w["blob"], w["lut"], 2, 128, indices_layout="idx4")
+    with pytest.raises(RuntimeError):
+        fx.qgemm_debug_simple(x, w["blob"], w["lut"], 4, 128)
+    with pytest.raises(RuntimeError):
+        fx.qgemm_dense(x, torch.zeros(256, 128, dtype=torch.float16))
+    with pytest.raises(ValueError):
+        fx.qgemm_gemv_mlp(x, torch.zeros(3, 15, dtype=torch.int64), torch.zeros(1, 256).half())
+    with pytest.raises(ValueError):
+        fx.qgemm_gemv_multi(x, torch.zeros(2, 14, dtype=torch.int64))
+
+
+def test_gates_and_tables():
+    assert fx.gemv_stream_available() and fx.gemv_splitk_available() and fx.gemv_mlp_available()
+    assert fx.gemv_multi_available() and fx.dual_stream_available()
+    assert fx.gemv_splitk_fht_available() and fx.gemv_fht_stream_available()
+    assert len(fx.GEMV_SPLITK_PAIRS) == 20 and (4, 0) in fx.GEMV_STREAM_PAIRS
+    assert fx.GEMV_SPLITK_MAX_RESIDUAL_RANK == 256 and fx.DUAL_STREAM_MAX_M == 16
+    assert fx.gemv_splitk_supported(4, 0, 128, 12288, 4096, 1)
+    assert fx.gemv_splitk_supported(1, 4, 16, 4096, 12288, 1, 256)
+    assert not fx.gemv_splitk_supported(4, 0, 128, 12288, 4096, 2)          # M != 1
+    assert not fx.gemv_splitk_supported(4, 0, 128, 12288, 4096, 1, 300)     # rank cap
+    assert not fx.gemv_splitk_supported(4, 0, 48, 12288, 4096, 1)
+    assert not fx.gemv_splitk_supported(4, 0, 128, 12200, 4096, 1)
+    assert not fx.gemv_stream_supported(4, 4, 128, 4096, 4096, 1)           # pair table
+    assert not fx.gemv_stream_supported(4, 0, 32, 4096, 4096, 1)            # gs table
+    assert fx.gemv_splitk_fht_supported(4, 0, 128, 4096, 12288, 1)
+    assert not fx.gemv_splitk_fht_supported(4, 0, 128, 4096, 32768, 1)      # segment > 16384
+    assert fx.gemv_mlp_supported(4096, 12288, [(4, 0, 128), (4, 1, 128)])
+    assert not fx.gemv_mlp_supported(4096, 12288, [(4, 0, 128)])
+    assert fx.gemv_multi_supported(4096, 48, [(4, 0, 128), (3, 3, 64)])
+    assert fx.dual_stream_supported(4, 0, 128, 4096, 4096)
+    assert not fx.dual_stream_supported(4, 0, 128, 4000, 4096)
+    # the split policy: wide outputs need no split, narrow ones split K
+    assert fx.gemv_split_hint(12288, 4096) == 1 and fx.gemv_split_hint(248320, 4096) == 1
+    for N in (1024, 512, 128):
+        s = fx.gemv_split_hint(N, 4096)
+        assert s > 1 and 64 % s == 0
+    assert 0 < _C.gemv_lds_bytes(12288, 4096, 4, 0, 128) <= fx.LDS_BYTES_PER_CU
+
+
+def test_fht_module_surface():
+    assert fht.segments(12288) == [(0, 8192), (8192, 4096)]
+    signs = fht.rotation_signs(256, 11)
+    assert torch.equal(signs, O.rotation_signs(256, 11))
+    x = make_x(4, 256, dtype=torch.float32)
+    assert torch.equal(fht.fht_apply(x, signs, backend="reference"), O.fht_reference(x, signs))
+    assert torch.equal(fht.fht_adjoint(x, signs, backend="reference"),
+                       O.fht_adjoint_reference(x, signs))
+    T = fht.build_rotation_matrix(256, 11)
+    assert np.allclose(T.double().numpy(), O.rotation_matrix(signs), atol=1e-7)
+    assert (fht.fht_apply(x, signs, backend="matmul") - x @ T).abs().max() < 1e-5
+    s = torch.rand(256) + 0.5
+    assert torch.equal(fht.fht_apply_awq(x, signs, s, backend="reference"),
+                       O.fht_awq_reference(x, signs, s))
+    with pytest.raises(RuntimeError):
+        fht.fht_apply(x, signs, backend="kernel")                   # CPU tensor
+    with pytest.raises(ValueError):
+        fht.fht_apply(x, signs, backend="nope")
+    with pytest.raises(ValueError):
+        fht.fht_apply(x, signs[:-1])
+    y = x.clone()
+    fht.fht_apply_(y, signs, backend="reference")
+    assert torch.equal(y, O.fht_reference(x, signs))
+    xa = x.clone().requires_grad_(True)
+    g = make_x(4, 256, seed=9, dtype=torch.float32)
+    fht.fht_apply(xa, signs, backend="reference").backward(g)
+    assert torch.equal(xa.grad, O.fht_adjoint_reference(g, signs))
+
+
+def test_module_layer_reference_mode_matches_oracle():
+    N, K = 256, 128
+    w = make_weight(N, K, 4, 64, seed=3, bits2=2, rank=8, bias=True, act_dtype=torch.float32)
+    m = pm.PalettizedLinear(w["blob"], w["lut"], 4, 64, N, K, bias=w["bias"], resA=w["resA"],
+                            resB=w["resB"], indices2=w["blob2"], lut2=w["lut2"], bitwidth2=2,
+                            reference=True, rotation_seed=5, rotation_k=K)
+    x = make_x(2, K, dtype=torch.float32).reshape(1, 2, K)
+    ref = O.linear_reference(x, w["blob"], w["lut"], N, K, 64, 4, w["blob2"], w["lut2"], 2,
+                             w["resA"], w["resB"], w["bias"], signs=O.rotation_signs(K, 5))
+    assert torch.equal(m(x), ref) and m(x).shape == (1, 2, N)
+    m._cache_logical_indices()
+    assert torch.equal(m(x), ref)                                  # cached-index gather
+    assert torch.equal(pm.reference_dequant(w["blob"], w["lut"], N, K, 64, 4),
+                       O.dequant(w["blob"], w["lut"], N, K, 64, 4))
+
+
+def test_module_layer_constructor_contract():
+    w = make_weight(256, 128, 4, 128, seed=3)
+    mk = lambda **kw: pm.PalettizedLinear(kw.pop("indices", w["blob"]), w["lut"],
+                                          kw.pop("bitwidth", 4), 128, kw.pop("N", 256),
+                                          kw.pop("K", 128), **kw)
+    mk()
+    with pytest.raises(ValueError):
+        mk(N=200, indices=torch.zeros(200 * 64, dtype=torch.uint8))   # kernel mode needs N%128
+    mk(N=200, indices=torch.zeros(200 * 64, dtype=torch.uint8), reference=True)
+    with pytest.raises(ValueError):
+        mk(indices=w["blob"][:-1])
+    with pytest.raises(ValueError):
+        mk(bitwidth=5)
+    with pytest.raises(ValueError):
+        mk(indices2=w["blob"])                                        # half a second stream
+    with pytest.raises(ValueError):
+        mk(awq_scale=torch.ones(128))                                 # awq without rotation
+    with pytest.raises(ValueError):
+        mk(rotation_seed=1, rotation_k=64)
+    with pytest.raises(ValueError):
+        mk(rotation_seed=1, rotation_k=128, awq_scale=-torch.ones(128))
+    with pytest.raises(ValueError):
+        mk(resA=torch.zeros(256, 4), resB=torch.zeros(5, 128))
+    m = mk(rotation_seed=1, rotation_k=128, awq_scale=torch.ones(128))
+    assert m.fold_order == "rotate_then_awq"
+    # kernel mode on CPU tensors fails loudly instead of computing in torch
+    with pytest.raises(RuntimeError):
+        mk()(make_x(1, 128))
+
+
+def test_fused_mlp_falls_through_on_unfusable_inputs():
+    wg, wu = make_weight(256, 128, seed=1), make_weight(256, 128, seed=2)
+    wd = make_weight(128, 256, seed=3)
+    g = pm.PalettizedLinear(wg["blob"], wg["lut"], 4, 128, 256, 128, reference=True)
+    u = pm.PalettizedLinear(wu["blob"], wu["lut"], 4, 128, 256, 128, reference=True)
+    d = pm.PalettizedLinear(wd["blob"], wd["lut"], 4, 128, 128, 256, reference=True)
+    mlp = pm.FusedPalettizedMLP(g, u, d, torch.nn.functional.silu)
+    x = make_x(1, 128, dtype=torch.float32)
+    y = mlp(x)
+    ref = O.mlp_reference(x, *[dict(blob=w["blob"], lut=w["lut"], N=w["N"], K=w["K"],
+                                    group_size=128, bits=4) for w in (wg, wu, wd)])
+    assert torch.equal(y, ref)
+    assert mlp._merge_state is None                                 # fp32 input: never built
+    assert mlp._build_state(torch.device("cpu"), torch.float16)["reason"] == "reference member"

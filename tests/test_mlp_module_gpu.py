@@ -1,0 +1,154 @@
+"""GPU parity of the merged gate/up launch, the grouped launch, the MLP block
+and the module layer's kernel mode against the oracle / the reference mode."""
+import ctypes
+
+import pytest
+import torch
+
+import flute_extended as fx
+import flute_oracle as O
+import palettized_modules as pm
+from flute_extended import _lib
+from _util import make_weight, make_x, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-3
+
+
+def _row(w, out=None, signs=None, awq=None):
+    p = lambda t: 0 if t is None else t.data_ptr()
+    return [p(w["blob_d"]), p(w["lut_d"]), p(w.get("blob2_d")), p(w.get("lut2_d")),
+            p(w.get("resB_d")), p(w.get("resA_d")), p(w.get("bias_d")), p(out), w["N"],
+            0 if w["resB"] is None else w["resB"].shape[0], w["bits"], w["bits2"], w["gs"],
+            p(signs), p(awq)]
+
+
+def _exact(w, x):
+    return O.linear_exact(x, w["blob"].numpy(), w["lut"], w["N"], w["K"], w["gs"], w["bits"],
+                          w["blob2"].numpy() if w["bits2"] else None, w["lut2"], w["bits2"],
+                          w["resA"], w["resB"], w["bias"])
+
+
+@pytest.mark.parametrize("gspec,uspec", [
+    (dict(bits=4), dict(bits=4)),
+    (dict(bits=4, bits2=1, gs=64), dict(bits=1, bits2=4, rank=8, bias=True)),
+    (dict(bits=3, gs=32), dict(bits=2, rank=4)),
+])
+def test_merged_gate_up_silu(gspec, uspec):
+    N, K = 1024, 2048
+    g = make_weight(N, K, seed=1, device=DEV, **gspec)
+    u = make_weight(N, K, seed=2, device=DEV, **uspec)
+    x = make_x(1, K, seed=3)
+    out = torch.zeros(1, N, dtype=torch.float16, device=DEV)
+    table = torch.tensor([_row(g), _row(u)], dtype=torch.int64)
+    y = fx.qgemm_gemv_mlp(x.to(DEV), table, out)
+    assert y.data_ptr() == out.data_ptr()
+    ref = O.silu_mul_exact(_exact(g, x), _exact(u, x)).half()
+    assert rel_l2(y.cpu(), ref) <= TOL
+    y1 = y.clone()
+    fx.qgemm_gemv_mlp(x.to(DEV), table, out)
+    assert torch.equal(out, y1)
+
+
+def test_merged_gate_up_with_different_rotations():
+    N, K = 512, 4096
+    g = make_weight(N, K, seed=1, device=DEV)
+    u = make_weight(N, K, seed=2, device=DEV)
+    x = make_x(1, K, seed=3)
+    sg, su = O.rotation_signs(K, 1).to(DEV), O.rotation_signs(K, 2).to(DEV)
+    out = torch.zeros(1, N, dtype=torch.float16, device=DEV)
+    table = torch.tensor([_row(g, signs=sg), _row(u, signs=su)], dtype=torch.int64)
+    y = fx.qgemm_gemv_mlp(x.to(DEV), table, out).cpu()
+    ref = O.silu_mul_exact(_exact(g, O.fht_reference(x, sg.cpu())),
+                           _exact(u, O.fht_reference(x, su.cpu()))).half()
+    assert rel_l2(y, ref) <= TOL
+
+
+def test_grouped_launch():
+    K = 2048
+    ws = [make_weight(512, K, seed=1, device=DEV),
+          make_weight(256, K, bits=3, gs=64, bits2=3, rank=8, seed=2, device=DEV),
+          make_weight(128, K, bits=2, gs=32, bias=True, seed=3, device=DEV)]
+    outs = [torch.zeros(1, w["N"], dtype=torch.float16, device=DEV) for w in ws]
+    x = make_x(1, K, seed=4)
+    table = torch.tensor([_row(w, o) for w, o in zip(ws, outs)], dtype=torch.int64)
+    assert fx.qgemm_gemv_multi(x.to(DEV), table) is None
+    for w, o in zip(ws, outs):
+        assert rel_l2(o.cpu(), _exact(w, x).half()) <= TOL
+
+
+def _desc(w):
+    d = _lib.FluteLinear()
+    d.q1, d.lut1 = w["blob_d"].data_ptr(), w["lut_d"].data_ptr()
+    d.q1_bytes = w["blob_d"].numel()
+    d.N, d.K, d.b1, d.group_size = w["N"], w["K"], w["bits"], w["gs"]
+    d.lut_rows = w["lut"].shape[0]
+    d.lut_dtype = _lib.F16 if w["lut"].dtype == torch.float16 else _lib.BF16
+    return d
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_mlp_block_through_the_c_abi(dtype):
+    """Benchmark configuration 2 at full size: gate/up 4096 -> 12288, SiLU*mul,
+    down 12288 -> 4096, called straight through flute_mlp_block."""
+    H, I = 4096, 12288
+    g = make_weight(I, H, seed=1, device=DEV)
+    u = make_weight(I, H, seed=2, device=DEV)
+    d = make_weight(H, I, seed=3, device=DEV)
+    x = make_x(1, H, seed=4, dtype=dtype)
+    xd = x.to(DEV)
+    h = torch.zeros(1, I, dtype=dtype, device=DEV)
+    y = torch.zeros(1, H, dtype=dtype, device=DEV)
+    dg, du, dd = _desc(g), _desc(u), _desc(d)
+    act = _lib.F16 if dtype == torch.float16 else _lib.BF16
+    st = _lib.lib.flute_mlp_block(ctypes.byref(dg), ctypes.byref(du), ctypes.byref(dd),
+                                  xd.data_ptr(), h.data_ptr(), y.data_ptr(), act,
+                                  torch.cuda.current_stream().cuda_stream)
+    assert st == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    h_ref = O.silu_mul_exact(_exact(g, x), _exact(u, x)).to(dtype)
+    tol = TOL if dtype == torch.float16 else 4e-3      # bf16: the output rounding alone is 2^-9
+    assert rel_l2(h.cpu(), h_ref) <= tol
+    assert rel_l2(y.cpu(), _exact(d, h.cpu()).to(dtype)) <= tol
+
+
+def _modules(w, **kw):
+    args = dict(bias=w["bias"], resA=w["resA"], resB=w["resB"], indices2=w["blob2"],
+                lut2=w["lut2"], bitwidth2=w["bits2"] or None)
+    args.update(kw)
+    ref = pm.PalettizedLinear(w["blob"], w["lut"], w["bits"], w["gs"], w["N"], w["K"],
+                              reference=True, **args)
+    ker = pm.PalettizedLinear(w["blob"], w["lut"], w["bits"], w["gs"], w["N"], w["K"],
+                              reference=False, **args).to(DEV)
+    return ref, ker
+
+
+@pytest.mark.parametrize("spec", [dict(), dict(bits2=2, rank=8, bias=True), dict(bits=3, gs=32)])
+@pytest.mark.parametrize("rot", [False, True])
+def test_module_kernel_mode_matches_reference_mode_m1(spec, rot):
+    N, K = 512, 1024
+    w = make_weight(N, K, seed=5, **spec)
+    kw = dict(rotation_seed=9, rotation_k=K) if rot else {}
+    ref, ker = _modules(w, **kw)
+    x = make_x(1, K, seed=6)
+    pm.ROUTE_CENSUS.clear()
+    y = ker(x.to(DEV).reshape(1, 1, K))
+    assert y.shape == (1, 1, N)
+    assert rel_l2(y.cpu().reshape(1, N), ref(x)) <= TOL
+    assert list(pm.ROUTE_CENSUS) == ["gemv_splitk_fht" if rot else "gemv_splitk"]
+
+
+def test_fused_mlp_module():
+    H, I = 1024, 2048
+    wg, wu, wd = (make_weight(I, H, seed=1), make_weight(I, H, seed=2, bits2=1),
+                  make_weight(H, I, seed=3))
+    refs, kers = zip(*[_modules(w) for w in (wg, wu, wd)])
+    act = torch.nn.functional.silu
+    mref = pm.FusedPalettizedMLP(*refs, act)
+    mker = pm.FusedPalettizedMLP(*kers, act)
+    x = make_x(1, H, seed=7)
+    pm.ROUTE_CENSUS.clear()
+    y = mker(x.to(DEV))
+    assert pm.ROUTE_CENSUS.get("gemv_mlp") == 1 and mker._merge_state["ok"]
+    assert rel_l2(y.cpu(), mref(x)) <= 2e-3       # two 16-bit roundings (h, then y) on each side
