@@ -1,0 +1,231 @@
+#!/usr/bin/env python3
+"""Benchmark of the idxN LUT-palettized decode path on one MI355X.
+
+One step = one token through the fused MLP block of the benchmark's second
+configuration: gate and up projections 4096 -> 12288 (one merged launch with
+the SiLU*mul epilogue), then the down projection 12288 -> 4096; idx4 blobs,
+group 128, fp16 LUTs, bf16 activations, M = 1.  The weights of a step live in
+HBM before the clock starts; consecutive steps use different weight sets whose
+total size exceeds three times the 256 MB Infinity Cache, so every step streams
+its 72 MiB from HBM.
+
+Prints ONE JSON line.  `value` is algorithmic bytes (packed indices + LUTs +
+activations in and out) per second over exactly `--steps` steps, timed with
+events on the stream the kernels run on.  `roofline` describes the dominant
+kernel (the merged gate+up GEMV) from a second timed region that launches only
+that kernel; `cpu_baseline` times the oracle's restatement of the upstream
+torch path on the host for a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path[:0] = [os.path.join(ROOT, "rag-cache-engineering-qwen35-9b-flute_amd")]
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+MFMA_PEAK_TFLOPS = 2500.0      # MI355X published dense bf16/fp16 MFMA rate
+H, I, GS = 4096, 12288, 128
+
+
+def _weights(torch, N, K, gen, dev, lut_dtype):
+    """A synthetic idx4 weight: uniform random blob bytes are uniform indices (the
+    blob is a permutation of the logical nibbles); LUT ~ N(0, 0.02) sorted ascending."""
+    blob = torch.randint(0, 256, (N * K // 2,), dtype=torch.uint8, device=dev, generator=gen)
+    lut = (torch.randn(N // GS, 16, device=dev, generator=gen) * 0.02).sort(dim=1).values
+    return blob, lut.to(lut_dtype).contiguous()
+
+
+def _desc(_lib, blob, lut, N, K):
+    d = _lib.FluteLinear()
+    d.q1, d.lut1, d.q1_bytes = blob.data_ptr(), lut.data_ptr(), blob.numel()
+    d.N, d.K, d.b1, d.group_size, d.lut_rows = N, K, 4, GS, lut.shape[0]
+    d.lut_dtype = _lib.F16 if str(lut.dtype) == "torch.float16" else _lib.BF16
+    return d
+
+
+def _time_graph(torch, fn, reps=3):
+    """Capture fn() (a sequence of launches on the current stream) once, replay it
+    `reps` times, return the best elapsed milliseconds of one replay."""
+    fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1))
+    return best
+
+
+def _cpu_baseline(torch, seconds_budget=20.0):
+    """The upstream reference path as shipped (unpack the blob, gather the LUT,
+    fp32 matmul; scripts/palettized_modules.py:811-824, 1241-1251 upstream) through
+    the oracle, on the benchmark's first configuration: M=1, 4096 -> 4096, fp16."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import flute_oracle as O
+    from flute_extended import idxN
+    N = K = 4096
+    g = torch.Generator().manual_seed(0)
+    idx = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
+    blob = idxN.pack_idxn(idx.numpy(), 4)
+    lut = (torch.randn(N // GS, 16, generator=g) * 0.02).sort(dim=1).values.half()
+    x = torch.randn(1, K, generator=g).half()
+    O.linear_reference(x, blob, lut, N, K, GS, 4)
+    times = []
+    t_end = time.perf_counter() + seconds_budget
+    while len(times) < 10 and (time.perf_counter() < t_end or len(times) < 3):
+        t0 = time.perf_counter()
+        O.linear_reference(x, blob, lut, N, K, GS, 4)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    nbytes = N * K // 2 + lut.numel() * 2 + K * 2 + N * 2
+    return {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"M=1 4096->4096 idx4 gs128 fp16, as shipped (unpack+gather+fp32 matmul per "
+                      f"call), median of {len(times)} calls, {med * 1e3:.1f} ms/call, "
+                      f"os.cpu_count={os.cpu_count()}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=240)
+    ap.add_argument("--warmup", type=int, default=24)
+    ap.add_argument("--sets", type=int, default=12, help="distinct weight sets (72 MiB each)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N "
+              "without any exchange, see DESIGN.md)", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    from flute_extended import _lib          # fails loudly if libflute_hip.so is missing
+    import ctypes
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    act = torch.bfloat16
+
+    sets = []
+    for _ in range(args.sets):
+        g, u, d = (_weights(torch, I, H, gen, dev, torch.float16),
+                   _weights(torch, I, H, gen, dev, torch.float16),
+                   _weights(torch, H, I, gen, dev, torch.float16))
+        sets.append(dict(t=(g, u, d), g=_desc(_lib, *g, I, H), u=_desc(_lib, *u, I, H),
+                         d=_desc(_lib, *d, H, I)))
+    x = torch.randn(1, H, device=dev, generator=gen).to(act)
+    h = torch.zeros(1, I, dtype=act, device=dev)
+    y = torch.zeros(1, H, dtype=act, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def block(s):
+        st = _lib.lib.flute_mlp_block(ctypes.byref(s["g"]), ctypes.byref(s["u"]),
+                                      ctypes.byref(s["d"]), x.data_ptr(), h.data_ptr(),
+                                      y.data_ptr(), _lib.BF16,
+                                      torch.cuda.current_stream().cuda_stream)
+        if st != 0:
+            raise RuntimeError(_lib.last_error())
+
+    def gate_up(s):
+        st = _lib.lib.flute_gemv_mlp(ctypes.byref(s["g"]), ctypes.byref(s["u"]), x.data_ptr(),
+                                     h.data_ptr(), _lib.BF16, 0,
+                                     torch.cuda.current_stream().cuda_stream)
+        if st != 0:
+            raise RuntimeError(_lib.last_error())
+
+    # ---- parity gate on the first set (a row whose check failed is never reported) ----
+    block(sets[0])
+    torch.cuda.synchronize()
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import flute_oracle as O
+    (gb, gl), (ub, ul), (db, dl) = sets[0]["t"]
+
+    def oracle_rows(blob, lut, K, tile):
+        # the 128 rows of one tile, dequantised by the oracle from the blob bytes
+        per = (K // 64) * 4096
+        sub = blob[tile * per:(tile + 1) * per].cpu().numpy()
+        return O.dequant(sub, lut[tile:tile + 1].cpu(), 128, K, GS, 4).double()
+
+    xd = x.cpu().double()
+    hd = h.cpu().double()
+    num = den = 0.0
+    for tile in (0, 37, 95):
+        g_ = xd @ oracle_rows(gb, gl, H, tile).t()
+        u_ = xd @ oracle_rows(ub, ul, H, tile).t()
+        ref = O.silu_mul_exact(g_, u_)
+        got = hd[:, tile * 128:(tile + 1) * 128]
+        num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
+    err_h = (num / den) ** 0.5
+    num = den = 0.0
+    for tile in (0, 13, 31):
+        ref = hd @ oracle_rows(db, dl, I, tile).t()
+        got = y.cpu().double()[:, tile * 128:(tile + 1) * 128]
+        num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
+    err_y = (num / den) ** 0.5
+    parity_ok = err_h < 4e-3 and err_y < 4e-3          # bf16 outputs: rounding alone is 2^-9
+    if not parity_ok:
+        print(f"bench.py: parity gate failed (h {err_h:.2e}, y {err_y:.2e})", file=sys.stderr)
+        return 1
+
+    # ---- timed region 1: whole MLP blocks ------------------------------------------
+    for i in range(args.warmup):
+        block(sets[i % args.sets])
+    torch.cuda.synchronize()
+    ms_total = _time_graph(torch, lambda: [block(sets[i % args.sets]) for i in range(args.steps)])
+    ms_step = ms_total / args.steps
+
+    # ---- timed region 2: the dominant kernel alone ----------------------------------
+    ms_gu = _time_graph(torch, lambda: [gate_up(sets[i % args.sets])
+                                        for i in range(args.steps)]) / args.steps
+
+    lut_bytes = (I // GS) * 16 * 2
+    bytes_gate_up = 2 * (I * H // 2 + lut_bytes) + H * 2 + I * 2
+    bytes_down = H * I // 2 + (H // GS) * 16 * 2 + I * 2 + H * 2
+    bytes_step = bytes_gate_up + bytes_down
+    value = bytes_step / (ms_step * 1e-3) / 1e9
+    achieved = bytes_gate_up / (ms_gu * 1e-3) / 1e9
+
+    out = {
+        "metric": "M=1 LUT-GEMV achieved HBM GB/s (% of peak); M=256 LUT-GEMM TFLOP/s (% MFMA)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 accumulate, f16 LUT, bf16 act",
+        "data": "synthetic",
+        "config": {"workload": "fused MLP decode M=1: gate+up 4096->12288 (merged, SiLU*mul) + "
+                               "down 12288->4096, idx4, group 128, fp16 LUT, bf16 activations",
+                   "weight_sets": args.sets, "bytes_per_step": bytes_step,
+                   "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+                   "timing": "hipGraph replay, events on the launch stream",
+                   "parity_rel_l2": {"h": err_h, "y": err_y}},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "gemv4_kernel (merged gate+up, SiLU*mul)",
+                     "us_per_launch": round(ms_gu * 1e3, 3),
+                     "algorithmic_bytes_per_launch": bytes_gate_up},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = _cpu_baseline(torch)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())
