@@ -110,7 +110,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N "
-              "without any exchange, see DESIGN.md)", file=sys.stderr)
+              "without any exchange between devices)", file=sys.stderr)
         return 2
 
     import torch
