@@ -1,14 +1,184 @@
-// Small-M / prefill LUT GEMM (placeholder entry until the MFMA kernel lands in
-// this file): refuses loudly.
+// Host side of the small-M / prefill LUT GEMM: shape policy, workspace layout,
+// pre-passes (activation permutation, residual coefficients) and the launch.
+#include <stdlib.h>
+
+#include "gemm_kernel.h"
 #include "host_common.h"
+
+namespace flute {
+
+namespace {
+
+struct GemmShape {
+    int mb, kw, mw;       // 16-row blocks per wavefront, k ways, m ways
+    int wg_per_cu;        // workgroups the policy expects to be resident per CU
+};
+
+// M <= 16: one block, eight k ways (the launch is a weight stream, like the GEMV).
+// M <= 64: four blocks, eight k ways.  Larger: 128 rows of A per workgroup, two m
+// groups of four blocks, four k ways; further rows go to gridDim.y.
+GemmShape choose_gemm_shape(int M) {
+    if (M <= 16) return {1, 8, 1, 2};
+    if (M <= 64) return {4, 8, 1, 1};
+    return {4, 4, 2, 1};
+}
+
+template <int MB, int KW, int MW, bool BF16, int B1>
+flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
+    static bool attr_done = false;
+    if (!attr_done) {
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            (int)kLdsPerCU));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL((gemm_kernel<MB, KW, MW, BF16, B1>), grid, dim3(64 * KW * MW), lds, stream,
+                       p);
+    FLUTE_HIP_CHECK(hipGetLastError());
+    return FLUTE_OK;
+}
+
+template <int MB, int KW, int MW, bool BF16>
+flute_status launch_gemm_bits(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
+    if (p.nstreams == 1) {
+        switch (p.bits[0]) {
+            case 4: return launch_gemm<MB, KW, MW, BF16, 4>(p, grid, lds, stream);
+            case 3: return launch_gemm<MB, KW, MW, BF16, 3>(p, grid, lds, stream);
+            case 2: return launch_gemm<MB, KW, MW, BF16, 2>(p, grid, lds, stream);
+            default: return launch_gemm<MB, KW, MW, BF16, 1>(p, grid, lds, stream);
+        }
+    }
+    return launch_gemm<MB, KW, MW, BF16, 0>(p, grid, lds, stream);
+}
+
+template <bool BF16>
+flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 grid, int lds,
+                               hipStream_t stream) {
+    if (s.mb == 1) return launch_gemm_bits<1, 8, 1, BF16>(p, grid, lds, stream);
+    if (s.mw == 1) return launch_gemm_bits<4, 8, 1, BF16>(p, grid, lds, stream);
+    return launch_gemm_bits<4, 4, 2, BF16>(p, grid, lds, stream);
+}
+
+}  // namespace
+
+}  // namespace flute
 
 using namespace flute;
 
 extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C, int M,
-                                   int64_t lda, int64_t ldc, int act_dtype, void *stream) {
-    (void)A; (void)C; (void)M; (void)lda; (void)ldc; (void)act_dtype; (void)stream;
+                                   int64_t lda, int64_t ldc, int act_dtype, void *stream_) {
     flute_status st = validate_linear(w, 1, "flute_gemm");
     if (st != FLUTE_OK) return st;
-    set_error("flute_gemm: not built yet");
-    return FLUTE_ERR_UNSUPPORTED;
+    FLUTE_REQUIRE(act_dtype == FLUTE_F16 || act_dtype == FLUTE_BF16, FLUTE_ERR_INVALID,
+                  "flute_gemm: activations must be float16 or bfloat16");
+    FLUTE_REQUIRE(M >= 0, FLUTE_ERR_INVALID, "flute_gemm: M must be >= 0 (got %d)", M);
+    if (M == 0) return FLUTE_OK;
+    FLUTE_REQUIRE(A != nullptr && C != nullptr, FLUTE_ERR_INVALID,
+                  "flute_gemm: A and C must not be NULL");
+    FLUTE_REQUIRE(lda >= w->K && ldc >= w->N, FLUTE_ERR_INVALID,
+                  "flute_gemm: row strides must cover a row (lda=%lld < K=%d or ldc=%lld < N=%d)",
+                  (long long)lda, w->K, (long long)ldc, w->N);
+    FLUTE_REQUIRE(((uintptr_t)A & 1) == 0 && ((uintptr_t)C & 1) == 0, FLUTE_ERR_INVALID,
+                  "flute_gemm: A and C must be 2-byte aligned");
+    FLUTE_REQUIRE(w->R == 0 || (int64_t)M * w->R <= 16384, FLUTE_ERR_UNSUPPORTED,
+                  "flute_gemm: the fused residual serves M*R <= 16384 (got M=%d, R=%d); add "
+                  "(A @ resB^T) @ resA^T outside for larger products",
+                  M, w->R);
+    hipStream_t stream = (hipStream_t)stream_;
+
+    GemmShape shape = choose_gemm_shape(M);
+    GemmParams p = {};
+    p.nstreams = w->b2 > 0 ? 2 : 1;
+    p.q[0] = (const uint8_t *)w->q1;
+    p.q[1] = (const uint8_t *)w->q2;
+    p.lut[0] = (const uint16_t *)w->lut1;
+    p.lut[1] = (const uint16_t *)w->lut2;
+    p.bits[0] = w->b1;
+    p.bits[1] = w->b2;
+    p.M = M;
+    p.N = w->N;
+    p.K = w->K;
+    p.G = w->K / 64;
+    p.gs = w->group_size;
+    p.lut_rows = w->lut_rows;
+    p.R = w->R;
+    p.resA = (const uint16_t *)w->resA;
+    p.bias = (const uint16_t *)w->bias;
+    p.C = C;
+    p.ldc = ldc;
+    p.out_bf16 = act_dtype == FLUTE_BF16;
+    p.vec_store = (ldc % 4 == 0) && (((uintptr_t)C & 7) == 0);
+    p.mblk_total = (M + 15) / 16;
+
+    // ---- pair tables: as much replication as the budget allows, 32 lanes at most ----
+    const int ngrp = w->group_size >= 128 ? 1 : 128 / w->group_size;
+    const int table_budget = (shape.mb == 1 ? 64 : 96) * 1024 / p.nstreams;
+    int lds_tables = 0;
+    for (int s = 0; s < p.nstreams; ++s) {
+        const int entries = ngrp << (2 * p.bits[s]);
+        int rl = 5;
+        while (rl > 0 && (entries << rl) * 4 > table_budget) --rl;
+        if (const char *e = getenv("FLUTE_GEMM_REP_LOG2")) rl = atoi(e) < rl ? atoi(e) : rl;
+        p.rep_log2[s] = rl;
+        p.tab_off[s] = lds_tables;
+        lds_tables += (entries << rl) * 4;
+    }
+    const int slot_bytes = shape.mb * 8 * 64 * 16;
+    const int lds_reduce = (shape.kw / 2) * shape.mw * slot_bytes;
+    const int lds = lds_tables > lds_reduce ? lds_tables : lds_reduce;
+    FLUTE_REQUIRE(lds <= kLdsPerCU, FLUTE_ERR_UNSUPPORTED,
+                  "flute_gemm: %d bytes of LDS exceed the %d of one CU", lds, kLdsPerCU);
+
+    // ---- grid and K split --------------------------------------------------------
+    const int tiles = w->N / 128;
+    const int mchunks = (p.mblk_total + shape.mb * shape.mw - 1) / (shape.mb * shape.mw);
+    const int64_t units = (int64_t)tiles * mchunks;
+    const int64_t cap = (int64_t)kNumCU * shape.wg_per_cu;
+    int ksplit = 1;
+    while (units * ksplit * 2 <= cap && p.G / (ksplit * 2) >= shape.kw) ksplit *= 2;
+    if (const char *e = getenv("FLUTE_GEMM_KSPLIT")) {
+        const int v = atoi(e);
+        if (v >= 1 && v <= p.G) ksplit = v;
+    }
+    p.gper = (p.G + ksplit - 1) / ksplit;
+    ksplit = (p.G + p.gper - 1) / p.gper;
+    p.ksplit = ksplit;
+    FLUTE_REQUIRE(mchunks <= 65535 && ksplit <= 65535, FLUTE_ERR_UNSUPPORTED,
+                  "flute_gemm: M=%d exceeds the grid", M);
+
+    // ---- workspace: [partial images][xb][Ap] -----------------------------------------
+    const size_t image = (size_t)shape.mw * shape.mb * 8 * 64 * 4;
+    const size_t p_floats = ksplit > 1 ? (size_t)ksplit * units * image : 0;
+    const size_t xb_floats = ((size_t)M * w->R + 3) & ~(size_t)3;
+    const size_t ap_floats = (size_t)p.G * 2 * p.mblk_total * 64 * 4;
+    float *base = nullptr;
+    int *tickets = nullptr;
+    st = get_workspace(p_floats + xb_floats + ap_floats + 64, (size_t)units + 1, stream, &base,
+                       &tickets);
+    if (st != FLUTE_OK) return st;
+    p.P = base;
+    p.tickets = tickets;
+    float *xb = base + p_floats;
+    u4_t *Ap = (u4_t *)(xb + xb_floats);
+    p.Ap = Ap;
+
+    {
+        const int64_t total = (int64_t)p.G * 2 * p.mblk_total * 64;
+        const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+        hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
+                           (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_total,
+                           (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16));
+        FLUTE_HIP_CHECK(hipGetLastError());
+    }
+    if (w->R > 0) {
+        hipLaunchKernelGGL(gemm_coeff_kernel, dim3(w->R, M), dim3(256), 0, stream,
+                           (const uint16_t *)A, lda, (const uint16_t *)w->resB, xb, w->K, w->R,
+                           p.out_bf16);
+        FLUTE_HIP_CHECK(hipGetLastError());
+        p.xb = xb;
+    }
+
+    const dim3 grid(tiles, mchunks, ksplit);
+    if (w->lut_dtype == FLUTE_BF16) return launch_gemm_shape<true>(shape, p, grid, lds, stream);
+    return launch_gemm_shape<false>(shape, p, grid, lds, stream);
 }

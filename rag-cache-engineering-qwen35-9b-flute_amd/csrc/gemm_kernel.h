@@ -1,0 +1,422 @@
+// LUT GEMM for M > 1 on the gfx950 matrix cores:  C[M, N] = A[M, K] @ W^T,
+// W[n, k] = LUT[n / gs][idx[n, k]], fp32 accumulate, one rounding.
+//
+// The weights never exist as a dense tile anywhere.  A lane loads one 16*b-byte
+// chunk of the idxN blob, which holds 8 rows x 16 k of one 128 x 64 tile, turns
+// the codes into 16-bit LUT values through a pair table in LDS (one lookup = two
+// weights) and feeds the result straight into v_mfma_f32_16x16x32 as the
+// row-side operand.  The blob's chunk order is the operand order of that
+// instruction up to a lane permutation:
+//
+//   MFMA lane l:  rho = l & 15 (operand row), kg = l >> 4 (k group of 8 values)
+//   chunk         th  = (rho >> 3) * 32 + (rho & 7) * 4 + kg     (wx, lane>>2, lane&3)
+//   operand (v, d, j), j = half of the 64-k tile:
+//       row  n = t*128 + wx*64 + v*16 + d*8 + (rho & 7)
+//       slot s = ktl*4 + s2*2 + e  ->  k = g*64 + (2j + ktl)*16 + 2*kg + 8*s2 + e
+//
+// so one chunk yields the 16 operands (v, d, j) of its 16 rows, and the
+// activations only have to present the same k order: a pre-pass writes them as
+// Ap[g][j][m / 16][lane = kg*16 + m % 16][8 values], one 16-byte load per operand.
+// The product is formed as C^T (rows of W on the MFMA row side), so a lane ends
+// up with four consecutive n of one m.
+//
+// Workgroup = KW x MW wavefronts on one 128-row tile: wavefront (kw, mw) walks the
+// k-tiles kw, kw + KW, ... for MB blocks of 16 rows of A.  Partial sums meet in a
+// tree through LDS, then (gridDim.z > 1) across workgroups through fp32 partials
+// and a ticket; the last arrival folds them in a fixed order.
+#pragma once
+
+#include "common.h"
+
+namespace flute {
+
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+
+struct GemmParams {
+    const uint8_t *q[2];
+    const uint16_t *lut[2];
+    const u4_t *Ap;        // permuted activations, LUT dtype, rows padded to 16
+    void *C;
+    const float *xb;       // [M, R] fp32 residual coefficients (A @ resB^T) or NULL
+    const uint16_t *resA;  // [N, R] activation dtype
+    const uint16_t *bias;  // [N] activation dtype
+    float *P;              // split-K partial images
+    int *tickets;
+    int64_t ldc;
+    int bits[2];
+    int tab_off[2];        // byte offset of each stream's pair tables in LDS
+    int rep_log2[2];       // log2 of the table replication (lanes per entry)
+    int nstreams;
+    int M, N, K, G, gs, lut_rows, R;
+    int mblk_total;        // padded M / 16
+    int ksplit, gper;      // gridDim.z and k-tiles per z slice
+    int out_bf16;          // dtype of C, resA, bias
+    int vec_store;         // C rows allow 8-byte stores
+};
+
+// Activation pre-pass: Ap[g][j][mb][lane][slot] in the LUT's 16-bit type.
+__global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t *Ap, int M,
+                                                        int64_t lda, int G, int mblk,
+                                                        int in_bf16, int out_bf16) {
+    const int64_t total = (int64_t)G * 2 * mblk * 64;
+    for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total;
+         o += (int64_t)gridDim.x * blockDim.x) {
+        const int lane = (int)(o & 63);
+        const int64_t rest = o >> 6;
+        const int mb = (int)(rest % mblk);
+        const int gj = (int)(rest / mblk);
+        const int g = gj >> 1, j = gj & 1;
+        const int m = mb * 16 + (lane & 15), kg = lane >> 4;
+        uint32_t out[4] = {0u, 0u, 0u, 0u};
+        if (m < M) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {              // s = ktl*2 + s2
+                const int k = g * 64 + (2 * j + (s >> 1)) * 16 + 2 * kg + 8 * (s & 1);
+                uint16_t a0 = A[m * lda + k], a1 = A[m * lda + k + 1];
+                if (in_bf16 != out_bf16) {
+                    a0 = round_act(in_bf16 ? bf2f(a0) : h2f(a0), out_bf16);
+                    a1 = round_act(in_bf16 ? bf2f(a1) : h2f(a1), out_bf16);
+                }
+                out[s] = (uint32_t)a0 | ((uint32_t)a1 << 16);
+            }
+        }
+        u4_t v = {out[0], out[1], out[2], out[3]};
+        Ap[o] = v;
+    }
+}
+
+// xb[m, r] = sum_k A[m, k] * resB[r, k] in fp32 (one workgroup per (r, m)).
+__global__ void __launch_bounds__(256) gemm_coeff_kernel(const uint16_t *A, int64_t lda,
+                                                         const uint16_t *resB, float *xb, int K,
+                                                         int R, int is_bf16) {
+    const int r = blockIdx.x, m = blockIdx.y;
+    float s = 0.0f;
+    for (int k = threadIdx.x; k < K; k += 256)
+        s = fmaf(load_act(A, m * lda + k, is_bf16), load_act(resB, (int64_t)r * K + k, is_bf16), s);
+    __shared__ float red[256];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) xb[(int64_t)m * R + r] = red[0];
+}
+
+__device__ __forceinline__ void gemm_ws_store(float *p, f4_t v) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        __hip_atomic_store(p + i, v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float gemm_ws_load(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <bool BF16>
+__device__ __forceinline__ f4_t mfma16(u4_t w, u4_t a, f4_t acc) {
+    if constexpr (BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, w),
+                                                       __builtin_bit_cast(bf8_t, a), acc, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8_t, w),
+                                                      __builtin_bit_cast(h8_t, a), acc, 0, 0, 0);
+}
+
+// The 2B-bit code of pair p of a chunk held as 4*B dwords (all indices constant
+// after unrolling).
+template <int B>
+__device__ __forceinline__ uint32_t pair_code(const uint32_t (&Q)[4 * B], int p) {
+    const int bit = 2 * B * p, dw = bit >> 5, sh = bit & 31;
+    if (sh + 2 * B <= 32) return __builtin_amdgcn_ubfe(Q[dw], sh, 2 * B);
+    return __builtin_amdgcn_alignbit(Q[dw + 1 < 4 * B ? dw + 1 : dw], Q[dw], sh) &
+           ((1u << (2 * B)) - 1u);
+}
+
+template <int B>
+__device__ __forceinline__ void load_chunk(uint32_t (&Q)[4 * B], const uint8_t *q, int64_t tile,
+                                           int th) {
+    const u4_t *src = (const u4_t *)(q + (tile * 64 + th) * (16 * B));
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+        const u4_t v = __builtin_nontemporal_load(src + i);
+        Q[4 * i + 0] = v[0];
+        Q[4 * i + 1] = v[1];
+        Q[4 * i + 2] = v[2];
+        Q[4 * i + 3] = v[3];
+    }
+}
+
+// One 64-k tile of one stream: 16 operands x MB MFMAs.
+//   lbase[v] : LDS byte address of this lane's column of the table that serves
+//              rows (wx, v) (the LUT group may depend on wx and v when gs < 128)
+template <int B, int MB, bool BF16>
+__device__ __forceinline__ void tile_mma(const uint32_t (&Q)[4 * B], const u4_t (&Ao)[MB][2],
+                                         f4_t (&acc)[MB][8], const uint32_t (&lbase)[4],
+                                         int code_shift) {
+    typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+#pragma unroll
+            for (int d = 0; d < 2; ++d) {
+                u4_t w;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {          // s = ktl*2 + s2
+                    const int p = (2 * j + (s >> 1)) * 16 + v * 4 + d * 2 + (s & 1);
+                    const uint32_t addr = (pair_code<B>(Q, p) << code_shift) + lbase[v];
+                    w[s] = *(LdsWord)addr;
+                }
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[mb][v * 2 + d] = mfma16<BF16>(w, Ao[mb][j], acc[mb][v * 2 + d]);
+            }
+        }
+    }
+}
+
+// B1 > 0: single stream of that width.  B1 == 0: widths read from the
+// parameters, one or two streams.
+template <int MB, int KW, int MW, bool BF16, int B1>
+__global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int NT = 64 * KW * MW;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kw = wave % KW, mw = wave / KW;
+    const int t = blockIdx.x;
+    const int mb0 = (blockIdx.y * MW + mw) * MB;       // first 16-row block of this wavefront
+    const int z = blockIdx.z;
+    const int rho = lane & 15, kg = lane >> 4;
+    const int wx = rho >> 3;
+    const int th = wx * 32 + (rho & 7) * 4 + kg;
+
+    // ---- pair tables ------------------------------------------------------------
+    const int ngrp = p.gs >= 128 ? 1 : 128 / p.gs;
+    for (int s = 0; s < p.nstreams; ++s) {
+        const int b = B1 > 0 ? B1 : p.bits[s];
+        const int rl = p.rep_log2[s];
+        const int total = ngrp << (2 * b + rl);
+        uint32_t *tab = (uint32_t *)(smem + p.tab_off[s]);
+        const uint16_t *lut = p.lut[s];
+        for (int i = tid; i < total; i += NT) {
+            const int code = (i >> rl) & ((1 << (2 * b)) - 1);
+            const int gl = i >> (rl + 2 * b);
+            int row = p.gs >= 128 ? (t * 128) / p.gs : t * ngrp + gl;
+            row = min(row, p.lut_rows - 1);
+            const uint16_t *lr = lut + ((size_t)row << b);
+            tab[i] = (uint32_t)lr[code & ((1 << b) - 1)] | ((uint32_t)lr[code >> b] << 16);
+        }
+    }
+    __syncthreads();
+
+    f4_t acc[MB][8];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[mb][i] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int gbeg = z * p.gper, gend = min(p.G, gbeg + p.gper);
+    const bool active = mb0 < p.mblk_total;            // whole wavefront
+    // Operand blocks past the padded M alias block 0; their sums are never stored.
+    int mbi[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) mbi[mb] = (mb0 + mb < p.mblk_total) ? mb0 + mb : 0;
+
+    auto load_a = [&](u4_t (&Ao)[MB][2], int g) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                Ao[mb][j] = p.Ap[(((int64_t)g * 2 + j) * p.mblk_total + mbi[mb]) * 64 + lane];
+    };
+    const uint32_t lds_base =
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    auto table_bases = [&](uint32_t (&lb)[4], int s, int b) {
+        const int rl = p.rep_log2[s];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int row = wx * 64 + v * 16;
+            const int gl = p.gs >= 128 ? 0 : row / p.gs;
+            lb[v] = lds_base + p.tab_off[s] +
+                    (((gl << (2 * b + rl)) + (lane & ((1 << rl) - 1))) << 2);
+        }
+    };
+
+    if (active) {
+        if constexpr (B1 > 0) {
+            uint32_t lb[4];
+            table_bases(lb, 0, B1);
+            const int cs = p.rep_log2[0] + 2;
+            uint32_t Qc[4 * B1], Qn[4 * B1];
+            u4_t Ac[MB][2], An[MB][2];
+            int g = gbeg + kw;
+            if (g < gend) {
+                load_chunk<B1>(Qc, p.q[0], (int64_t)t * p.G + g, th);
+                load_a(Ac, g);
+            }
+            while (g < gend) {
+                const int gn = g + KW;
+                const int gl = gn < gend ? gn : g;      // harmless reload on the last pass
+                load_chunk<B1>(Qn, p.q[0], (int64_t)t * p.G + gl, th);
+                load_a(An, gl);
+                tile_mma<B1, MB, BF16>(Qc, Ac, acc, lb, cs);
+#pragma unroll
+                for (int i = 0; i < 4 * B1; ++i) Qc[i] = Qn[i];
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    Ac[mb][0] = An[mb][0];
+                    Ac[mb][1] = An[mb][1];
+                }
+                g = gn;
+            }
+        } else {
+            for (int g = gbeg + kw; g < gend; g += KW) {
+                u4_t Ac[MB][2];
+                load_a(Ac, g);
+                for (int s = 0; s < p.nstreams; ++s) {
+                    uint32_t lb[4];
+                    const int cs = p.rep_log2[s] + 2;
+                    const int64_t tile = (int64_t)t * p.G + g;
+                    switch (p.bits[s]) {
+                        case 1: {
+                            uint32_t Q[4];
+                            table_bases(lb, s, 1);
+                            load_chunk<1>(Q, p.q[s], tile, th);
+                            tile_mma<1, MB, BF16>(Q, Ac, acc, lb, cs);
+                        } break;
+                        case 2: {
+                            uint32_t Q[8];
+                            table_bases(lb, s, 2);
+                            load_chunk<2>(Q, p.q[s], tile, th);
+                            tile_mma<2, MB, BF16>(Q, Ac, acc, lb, cs);
+                        } break;
+                        case 3: {
+                            uint32_t Q[12];
+                            table_bases(lb, s, 3);
+                            load_chunk<3>(Q, p.q[s], tile, th);
+                            tile_mma<3, MB, BF16>(Q, Ac, acc, lb, cs);
+                        } break;
+                        default: {
+                            uint32_t Q[16];
+                            table_bases(lb, s, 4);
+                            load_chunk<4>(Q, p.q[s], tile, th);
+                            tile_mma<4, MB, BF16>(Q, Ac, acc, lb, cs);
+                        } break;
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- tree over the KW wavefronts of one m group, through LDS ------------------
+    f4_t *red = (f4_t *)smem;                           // slot = [MB*8][64] f4
+    __syncthreads();                                    // tables are dead from here
+#pragma unroll
+    for (int step = KW / 2; step >= 1; step >>= 1) {
+        if (kw >= step && kw < 2 * step) {
+            f4_t *slot = red + (size_t)((kw - step) * MW + mw) * (MB * 8 * 64);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) slot[(mb * 8 + i) * 64 + lane] = acc[mb][i];
+        }
+        __syncthreads();
+        if (kw < step) {
+            const f4_t *slot = red + (size_t)(kw * MW + mw) * (MB * 8 * 64);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[mb][i] += slot[(mb * 8 + i) * 64 + lane];
+        }
+        __syncthreads();
+    }
+
+    // ---- across workgroups: partial images + ticket --------------------------------
+    if (p.ksplit > 1) {
+        const int unit = blockIdx.y * gridDim.x + blockIdx.x;       // (m chunk, n tile)
+        const size_t image = (size_t)MW * MB * 8 * 64 * 4;          // floats per unit per z
+        float *mine = p.P + ((size_t)z * gridDim.x * gridDim.y + unit) * image;
+        if (kw == 0) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    gemm_ws_store(mine + ((size_t)(mw * MB + mb) * 8 + i) * 256 + lane * 4,
+                                  acc[mb][i]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        int *flag = (int *)smem;
+        if (tid == 0) {
+            const int old = __hip_atomic_fetch_add(p.tickets + unit, 1, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+            *flag = (old == p.ksplit - 1);
+        }
+        __syncthreads();
+        if (!*flag) return;
+        if (kw == 0) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    f4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
+                    for (int zz = 0; zz < p.ksplit; ++zz) {
+                        const float *src = p.P +
+                                           ((size_t)zz * gridDim.x * gridDim.y + unit) * image +
+                                           ((size_t)(mw * MB + mb) * 8 + i) * 256 + lane * 4;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) s[r] += gemm_ws_load(src + r);
+                    }
+                    acc[mb][i] = s;
+                }
+        }
+        if (tid == 0)
+            __hip_atomic_store(p.tickets + unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // ---- epilogue: residual, bias, one rounding, store -------------------------------
+    if (kw != 0 || !active) return;
+    const int nb = t * 128 + (kg >> 1) * 64 + (kg & 1) * 4;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = (mb0 + mb) * 16 + rho;
+        if (mb0 + mb >= p.mblk_total || m >= p.M) continue;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int n0 = nb + (i >> 1) * 16 + (i & 1) * 8;
+            f4_t y = acc[mb][i];
+            if (p.R > 0) {
+                const float *xr = p.xb + (size_t)m * p.R;
+                for (int r = 0; r < p.R; ++r) {
+                    const float c = xr[r];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        y[e] = fmaf(c, load_act(p.resA, (int64_t)(n0 + e) * p.R + r, p.out_bf16),
+                                    y[e]);
+                }
+            }
+            if (p.bias) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] += load_act(p.bias, n0 + e, p.out_bf16);
+            }
+            uint16_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = round_act(y[e], p.out_bf16);
+            uint16_t *dst = (uint16_t *)p.C + (size_t)m * p.ldc + n0;
+            if (p.vec_store) {
+                uint2 pk;
+                pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+                pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+                *(uint2 *)dst = pk;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e] = o[e];
+            }
+        }
+    }
+}
+
+}  // namespace flute
