@@ -109,6 +109,7 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     p.out_bf16 = act_dtype == FLUTE_BF16;
     p.vec_store = (ldc % 4 == 0) && (((uintptr_t)C & 7) == 0);
     p.mblk_total = (M + 15) / 16;
+    if (const char *e = getenv("FLUTE_GEMM_DBG")) p.dbg = atoi(e);
 
     // ---- pair tables: as much replication as the budget allows, 32 lanes at most ----
     const int ngrp = w->group_size >= 128 ? 1 : 128 / w->group_size;

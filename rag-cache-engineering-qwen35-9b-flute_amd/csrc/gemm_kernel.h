@@ -55,6 +55,7 @@ struct GemmParams {
     int ksplit, gper;      // gridDim.z and k-tiles per z slice
     int out_bf16;          // dtype of C, resA, bias
     int vec_store;         // C rows allow 8-byte stores
+    int dbg;
 };
 
 // Activation pre-pass: Ap[g][j][mb][lane][slot] in the LUT's 16-bit type.
@@ -149,32 +150,46 @@ __device__ __forceinline__ void load_chunk(uint32_t (&Q)[4 * B], const uint8_t *
     }
 }
 
-// One 64-k tile of one stream: 16 operands x MB MFMAs.
+// The four lookups of operand (j, v, d).
+template <int B>
+__device__ __forceinline__ u4_t fetch_operand(const uint32_t (&Q)[4 * B], int j, int v, int d,
+                                              uint32_t lbase, int code_shift) {
+    typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
+    u4_t w;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {                      // s = ktl*2 + s2
+        const int p = (2 * j + (s >> 1)) * 16 + v * 4 + d * 2 + (s & 1);
+        const uint32_t addr = (pair_code<B>(Q, p) << code_shift) + lbase;
+        w[s] = *(LdsWord)addr;
+    }
+    return w;
+}
+
+// Half (32 k) of a 64-k tile of one stream: 8 operands x MB MFMAs.  The lookups
+// run one pair of operands ahead of the MFMAs that consume them, in two
+// alternating register sets, so the LDS latency hides behind matrix work.
 //   lbase[v] : LDS byte address of this lane's column of the table that serves
 //              rows (wx, v) (the LUT group may depend on wx and v when gs < 128)
 template <int B, int MB, bool BF16>
-__device__ __forceinline__ void tile_mma(const uint32_t (&Q)[4 * B], const u4_t (&Ao)[MB][2],
+__device__ __forceinline__ void half_mma(const uint32_t (&Q)[4 * B], int j, const u4_t (&Aj)[MB],
                                          f4_t (&acc)[MB][8], const uint32_t (&lbase)[4],
                                          int code_shift) {
-    typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
+    u4_t W[2][2];
+    W[0][0] = fetch_operand<B>(Q, j, 0, 0, lbase[0], code_shift);
+    W[0][1] = fetch_operand<B>(Q, j, 0, 1, lbase[0], code_shift);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-#pragma unroll
-            for (int d = 0; d < 2; ++d) {
-                u4_t w;
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {          // s = ktl*2 + s2
-                    const int p = (2 * j + (s >> 1)) * 16 + v * 4 + d * 2 + (s & 1);
-                    const uint32_t addr = (pair_code<B>(Q, p) << code_shift) + lbase[v];
-                    w[s] = *(LdsWord)addr;
-                }
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                    acc[mb][v * 2 + d] = mfma16<BF16>(w, Ao[mb][j], acc[mb][v * 2 + d]);
-            }
+    for (int v = 0; v < 4; ++v) {
+        if (v + 1 < 4) {
+            W[(v + 1) & 1][0] = fetch_operand<B>(Q, j, v + 1, 0, lbase[v + 1], code_shift);
+            W[(v + 1) & 1][1] = fetch_operand<B>(Q, j, v + 1, 1, lbase[v + 1], code_shift);
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int d = 0; d < 2; ++d)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                acc[mb][v * 2 + d] = mfma16<BF16>(W[v & 1][d], Aj[mb], acc[mb][v * 2 + d]);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -225,12 +240,10 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) mbi[mb] = (mb0 + mb < p.mblk_total) ? mb0 + mb : 0;
 
-    auto load_a = [&](u4_t (&Ao)[MB][2], int g) {
+    auto load_a = [&](u4_t (&Aj)[MB], int g, int j) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-                Ao[mb][j] = p.Ap[(((int64_t)g * 2 + j) * p.mblk_total + mbi[mb]) * 64 + lane];
+            Aj[mb] = p.Ap[(((int64_t)g * 2 + j) * p.mblk_total + mbi[mb]) * 64 + lane];
     };
     const uint32_t lds_base =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -251,31 +264,33 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             table_bases(lb, 0, B1);
             const int cs = p.rep_log2[0] + 2;
             uint32_t Qc[4 * B1], Qn[4 * B1];
-            u4_t Ac[MB][2], An[MB][2];
+            u4_t A0[MB], A1[MB];
             int g = gbeg + kw;
             if (g < gend) {
                 load_chunk<B1>(Qc, p.q[0], (int64_t)t * p.G + g, th);
-                load_a(Ac, g);
+                load_a(A0, g, 0);
+                load_a(A1, g, 1);
             }
             while (g < gend) {
                 const int gn = g + KW;
                 const int gl = gn < gend ? gn : g;      // harmless reload on the last pass
-                load_chunk<B1>(Qn, p.q[0], (int64_t)t * p.G + gl, th);
-                load_a(An, gl);
-                tile_mma<B1, MB, BF16>(Qc, Ac, acc, lb, cs);
+                load_chunk<B1>(Qn, p.q[0], (int64_t)t * p.G + ((p.dbg & 1) ? gbeg : gl), th);
+                __builtin_amdgcn_sched_barrier(0);
+                half_mma<B1, MB, BF16>(Qc, 0, A0, acc, lb, cs);
+                load_a(A0, (p.dbg & 2) ? gbeg : gl, 0);  // half a tile ahead of its use
+                __builtin_amdgcn_sched_barrier(0);
+                half_mma<B1, MB, BF16>(Qc, 1, A1, acc, lb, cs);
+                load_a(A1, (p.dbg & 2) ? gbeg : gl, 1);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < 4 * B1; ++i) Qc[i] = Qn[i];
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    Ac[mb][0] = An[mb][0];
-                    Ac[mb][1] = An[mb][1];
-                }
                 g = gn;
             }
         } else {
             for (int g = gbeg + kw; g < gend; g += KW) {
-                u4_t Ac[MB][2];
-                load_a(Ac, g);
+                u4_t A0[MB], A1[MB];
+                load_a(A0, g, 0);
+                load_a(A1, g, 1);
                 for (int s = 0; s < p.nstreams; ++s) {
                     uint32_t lb[4];
                     const int cs = p.rep_log2[s] + 2;
@@ -285,25 +300,29 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                             uint32_t Q[4];
                             table_bases(lb, s, 1);
                             load_chunk<1>(Q, p.q[s], tile, th);
-                            tile_mma<1, MB, BF16>(Q, Ac, acc, lb, cs);
+                            half_mma<1, MB, BF16>(Q, 0, A0, acc, lb, cs);
+                            half_mma<1, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
                         case 2: {
                             uint32_t Q[8];
                             table_bases(lb, s, 2);
                             load_chunk<2>(Q, p.q[s], tile, th);
-                            tile_mma<2, MB, BF16>(Q, Ac, acc, lb, cs);
+                            half_mma<2, MB, BF16>(Q, 0, A0, acc, lb, cs);
+                            half_mma<2, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
                         case 3: {
                             uint32_t Q[12];
                             table_bases(lb, s, 3);
                             load_chunk<3>(Q, p.q[s], tile, th);
-                            tile_mma<3, MB, BF16>(Q, Ac, acc, lb, cs);
+                            half_mma<3, MB, BF16>(Q, 0, A0, acc, lb, cs);
+                            half_mma<3, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
                         default: {
                             uint32_t Q[16];
                             table_bases(lb, s, 4);
                             load_chunk<4>(Q, p.q[s], tile, th);
-                            tile_mma<4, MB, BF16>(Q, Ac, acc, lb, cs);
+                            half_mma<4, MB, BF16>(Q, 0, A0, acc, lb, cs);
+                            half_mma<4, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
                     }
                 }
@@ -363,12 +382,22 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     f4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
-                    for (int zz = 0; zz < p.ksplit; ++zz) {
-                        const float *src = p.P +
-                                           ((size_t)zz * gridDim.x * gridDim.y + unit) * image +
-                                           ((size_t)(mw * MB + mb) * 8 + i) * 256 + lane * 4;
+                    const float *src = p.P + (size_t)unit * image +
+                                       ((size_t)(mw * MB + mb) * 8 + i) * 256 + lane * 4;
+                    const size_t zstride = (size_t)gridDim.x * gridDim.y * image;
+                    for (int z0 = 0; z0 < p.ksplit; z0 += 4) {     // 16 loads in flight
+                        float part[4][4];
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) s[r] += gemm_ws_load(src + r);
+                        for (int a = 0; a < 4; ++a)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                part[a][r] = (z0 + a < p.ksplit)
+                                                 ? gemm_ws_load(src + (z0 + a) * zstride + r)
+                                                 : 0.0f;
+#pragma unroll
+                        for (int a = 0; a < 4; ++a)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) s[r] += part[a][r];
                     }
                     acc[mb][i] = s;
                 }
