@@ -23,26 +23,39 @@ GemmShape choose_gemm_shape(int M) {
     return {4, 4, 2, 1};
 }
 
-template <int MB, int KW, int MW, bool BF16, int B1>
+template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false>
 flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
     static bool attr_done = false;
     if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1>,
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1, PERM>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
                                             (int)kLdsPerCU));
         attr_done = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<MB, KW, MW, BF16, B1>), grid, dim3(64 * KW * MW), lds, stream,
-                       p);
+    hipLaunchKernelGGL((gemm_kernel<MB, KW, MW, BF16, B1, PERM>), grid, dim3(64 * KW * MW), lds,
+                       stream, p);
     FLUTE_HIP_CHECK(hipGetLastError());
     return FLUTE_OK;
 }
 
+#ifdef FLUTE_GEMM_DEV_MINIMAL
+// Development builds: only the 4-bit fp16 M > 64 kernel, to keep compile time short.
+template <bool BF16>
+flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 grid, int lds,
+                               hipStream_t stream) {
+    if (!BF16 && s.mw == 2 && p.nstreams == 1 && p.bits[0] == 4 && p.rep_log2[0] == 6)
+        return launch_gemm<4, 4, 2, false, 4, true>(p, grid, lds, stream);
+    set_error("flute_gemm: development build without this kernel");
+    return FLUTE_ERR_UNSUPPORTED;
+}
+#else
 template <int MB, int KW, int MW, bool BF16>
 flute_status launch_gemm_bits(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
     if (p.nstreams == 1) {
         switch (p.bits[0]) {
-            case 4: return launch_gemm<MB, KW, MW, BF16, 4>(p, grid, lds, stream);
+            case 4:
+                if (p.rep_log2[0] == 6) return launch_gemm<MB, KW, MW, BF16, 4, true>(p, grid, lds, stream);
+                return launch_gemm<MB, KW, MW, BF16, 4>(p, grid, lds, stream);
             case 3: return launch_gemm<MB, KW, MW, BF16, 3>(p, grid, lds, stream);
             case 2: return launch_gemm<MB, KW, MW, BF16, 2>(p, grid, lds, stream);
             default: return launch_gemm<MB, KW, MW, BF16, 1>(p, grid, lds, stream);
@@ -58,6 +71,8 @@ flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 gri
     if (s.mw == 1) return launch_gemm_bits<4, 8, 1, BF16>(p, grid, lds, stream);
     return launch_gemm_bits<4, 4, 2, BF16>(p, grid, lds, stream);
 }
+
+#endif
 
 }  // namespace
 
@@ -107,26 +122,37 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     p.C = C;
     p.ldc = ldc;
     p.out_bf16 = act_dtype == FLUTE_BF16;
-    p.vec_store = (ldc % 4 == 0) && (((uintptr_t)C & 7) == 0);
+    p.vec_store = (ldc % 8 == 0) && (((uintptr_t)C & 15) == 0);
     p.mblk_total = (M + 15) / 16;
-    if (const char *e = getenv("FLUTE_GEMM_DBG")) p.dbg = atoi(e);
 
-    // ---- pair tables: as much replication as the budget allows, 32 lanes at most ----
+    // ---- pair tables ---------------------------------------------------------------
+    // A single 4-bit stream with at most two LUT groups per 128-row tile gets 64-lane
+    // replication (256 bytes per entry, 64 KB per group, first table at LDS offset 0:
+    // the layout the one-instruction address needs).  Everything else: as much
+    // replication as the budget allows, 32 lanes at most.
     const int ngrp = w->group_size >= 128 ? 1 : 128 / w->group_size;
+    const bool perm = p.nstreams == 1 && p.bits[0] == 4 && ngrp <= 2 &&
+                      getenv("FLUTE_GEMM_NO_PERM") == nullptr;
     const int table_budget = (shape.mb == 1 ? 64 : 96) * 1024 / p.nstreams;
     int lds_tables = 0;
     for (int s = 0; s < p.nstreams; ++s) {
         const int entries = ngrp << (2 * p.bits[s]);
         int rl = 5;
         while (rl > 0 && (entries << rl) * 4 > table_budget) --rl;
-        if (const char *e = getenv("FLUTE_GEMM_REP_LOG2")) rl = atoi(e) < rl ? atoi(e) : rl;
+        if (perm) rl = 6;
         p.rep_log2[s] = rl;
         p.tab_off[s] = lds_tables;
         lds_tables += (entries << rl) * 4;
     }
+    if (perm) {                                  // per-wavefront tile staging behind the tables
+        p.stage_off = lds_tables;
+        lds_tables += shape.kw * shape.mw * 4096;
+    }
     const int slot_bytes = shape.mb * 8 * 64 * 16;
     const int lds_reduce = (shape.kw / 2) * shape.mw * slot_bytes;
-    const int lds = lds_tables > lds_reduce ? lds_tables : lds_reduce;
+    const int lds_tile = shape.mw * shape.mb * 16 * 132 * 4 + 16;   // totals tile + ticket flag
+    int lds = lds_tables > lds_reduce ? lds_tables : lds_reduce;
+    if (lds_tile > lds) lds = lds_tile;
     FLUTE_REQUIRE(lds <= kLdsPerCU, FLUTE_ERR_UNSUPPORTED,
                   "flute_gemm: %d bytes of LDS exceed the %d of one CU", lds, kLdsPerCU);
 
@@ -134,6 +160,7 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     const int tiles = w->N / 128;
     const int mchunks = (p.mblk_total + shape.mb * shape.mw - 1) / (shape.mb * shape.mw);
     const int64_t units = (int64_t)tiles * mchunks;
+    p.mblk_pad = mchunks * shape.mb * shape.mw;
     const int64_t cap = (int64_t)kNumCU * shape.wg_per_cu;
     int ksplit = 1;
     while (units * ksplit * 2 <= cap && p.G / (ksplit * 2) >= shape.kw) ksplit *= 2;
@@ -151,7 +178,7 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     const size_t image = (size_t)shape.mw * shape.mb * 8 * 64 * 4;
     const size_t p_floats = ksplit > 1 ? (size_t)ksplit * units * image : 0;
     const size_t xb_floats = ((size_t)M * w->R + 3) & ~(size_t)3;
-    const size_t ap_floats = (size_t)p.G * 2 * p.mblk_total * 64 * 4;
+    const size_t ap_floats = (size_t)p.G * 2 * p.mblk_pad * 64 * 4;
     float *base = nullptr;
     int *tickets = nullptr;
     st = get_workspace(p_floats + xb_floats + ap_floats + 64, (size_t)units + 1, stream, &base,
@@ -164,10 +191,10 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     p.Ap = Ap;
 
     {
-        const int64_t total = (int64_t)p.G * 2 * p.mblk_total * 64;
+        const int64_t total = (int64_t)p.G * 2 * p.mblk_pad * 64;
         const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
         hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
-                           (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_total,
+                           (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
                            (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16));
         FLUTE_HIP_CHECK(hipGetLastError());
     }
@@ -179,6 +206,9 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
         p.xb = xb;
     }
 
+#ifdef FLUTE_GEMM_TRACE
+    if (const char *e = getenv("FLUTE_GEMM_TRACE_PTR")) p.trace = (unsigned long long *)strtoull(e, nullptr, 10);
+#endif
     const dim3 grid(tiles, mchunks, ksplit);
     if (w->lut_dtype == FLUTE_BF16) return launch_gemm_shape<true>(shape, p, grid, lds, stream);
     return launch_gemm_shape<false>(shape, p, grid, lds, stream);

@@ -49,13 +49,17 @@ struct GemmParams {
     int bits[2];
     int tab_off[2];        // byte offset of each stream's pair tables in LDS
     int rep_log2[2];       // log2 of the table replication (lanes per entry)
+    int stage_off;         // byte offset of the per-wavefront 4 KB tile staging buffers
     int nstreams;
     int M, N, K, G, gs, lut_rows, R;
-    int mblk_total;        // padded M / 16
+    int mblk_total;        // ceil(M / 16)
+    int mblk_pad;          // blocks Ap holds per half tile: gridDim.y * MW * MB
     int ksplit, gper;      // gridDim.z and k-tiles per z slice
     int out_bf16;          // dtype of C, resA, bias
-    int vec_store;         // C rows allow 8-byte stores
-    int dbg;
+    int vec_store;         // C rows allow 16-byte stores
+#ifdef FLUTE_GEMM_TRACE
+    unsigned long long *trace;   // [workgroup][16] timestamps, development builds only
+#endif
 };
 
 // Activation pre-pass: Ap[g][j][mb][lane][slot] in the LUT's 16-bit type.
@@ -107,14 +111,20 @@ __global__ void __launch_bounds__(256) gemm_coeff_kernel(const uint16_t *A, int6
     if (threadIdx.x == 0) xb[(int64_t)m * R + r] = red[0];
 }
 
-__device__ __forceinline__ void gemm_ws_store(float *p, f4_t v) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        __hip_atomic_store(p + i, v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 __device__ __forceinline__ float gemm_ws_load(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+
+#ifdef FLUTE_GEMM_TRACE
+#define GEMM_TRACE(slot)                                                                    \
+    do {                                                                                    \
+        if (p.trace && threadIdx.x == 0)                                                    \
+            p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + \
+                    (slot)] = wall_clock64();                                               \
+    } while (0)
+#else
+#define GEMM_TRACE(slot) do {} while (0)
+#endif
 
 template <bool BF16>
 __device__ __forceinline__ f4_t mfma16(u4_t w, u4_t a, f4_t acc) {
@@ -137,9 +147,8 @@ __device__ __forceinline__ uint32_t pair_code(const uint32_t (&Q)[4 * B], int p)
 }
 
 template <int B>
-__device__ __forceinline__ void load_chunk(uint32_t (&Q)[4 * B], const uint8_t *q, int64_t tile,
-                                           int th) {
-    const u4_t *src = (const u4_t *)(q + (tile * 64 + th) * (16 * B));
+__device__ __forceinline__ void load_chunk(uint32_t (&Q)[4 * B], const uint8_t *chunk) {
+    const u4_t *src = (const u4_t *)chunk;
 #pragma unroll
     for (int i = 0; i < B; ++i) {
         const u4_t v = __builtin_nontemporal_load(src + i);
@@ -150,8 +159,11 @@ __device__ __forceinline__ void load_chunk(uint32_t (&Q)[4 * B], const uint8_t *
     }
 }
 
-// The four lookups of operand (j, v, d).
-template <int B>
+// The four lookups of operand (j, v, d).  PERM (4-bit codes, 64-lane replication,
+// table on a 64 KB boundary of LDS): the code is a whole byte of the chunk and the
+// entry stride is 256 bytes, so one v_perm_b32 drops it into byte 1 of the lane's
+// column address.
+template <int B, bool PERM>
 __device__ __forceinline__ u4_t fetch_operand(const uint32_t (&Q)[4 * B], int j, int v, int d,
                                               uint32_t lbase, int code_shift) {
     typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
@@ -159,7 +171,13 @@ __device__ __forceinline__ u4_t fetch_operand(const uint32_t (&Q)[4 * B], int j,
 #pragma unroll
     for (int s = 0; s < 4; ++s) {                      // s = ktl*2 + s2
         const int p = (2 * j + (s >> 1)) * 16 + v * 4 + d * 2 + (s & 1);
-        const uint32_t addr = (pair_code<B>(Q, p) << code_shift) + lbase;
+        uint32_t addr;
+        if constexpr (PERM) {
+            static_assert(B == 4, "byte codes");
+            addr = __builtin_amdgcn_perm(Q[p >> 2], lbase, 0x03020000u | ((4u + (p & 3)) << 8));
+        } else {
+            addr = (pair_code<B>(Q, p) << code_shift) + lbase;
+        }
         w[s] = *(LdsWord)addr;
     }
     return w;
@@ -170,32 +188,39 @@ __device__ __forceinline__ u4_t fetch_operand(const uint32_t (&Q)[4 * B], int j,
 // alternating register sets, so the LDS latency hides behind matrix work.
 //   lbase[v] : LDS byte address of this lane's column of the table that serves
 //              rows (wx, v) (the LUT group may depend on wx and v when gs < 128)
-template <int B, int MB, bool BF16>
+template <int B, int MB, bool BF16, bool PERM = false>
 __device__ __forceinline__ void half_mma(const uint32_t (&Q)[4 * B], int j, const u4_t (&Aj)[MB],
                                          f4_t (&acc)[MB][8], const uint32_t (&lbase)[4],
                                          int code_shift) {
-    u4_t W[2][2];
-    W[0][0] = fetch_operand<B>(Q, j, 0, 0, lbase[0], code_shift);
-    W[0][1] = fetch_operand<B>(Q, j, 0, 1, lbase[0], code_shift);
+    constexpr int AHEAD = 1;                             // pairs of operands in flight
+    u4_t W[AHEAD + 1][2];
+#pragma unroll
+    for (int v = 0; v < AHEAD; ++v) {
+        W[v][0] = fetch_operand<B, PERM>(Q, j, v, 0, lbase[v], code_shift);
+        W[v][1] = fetch_operand<B, PERM>(Q, j, v, 1, lbase[v], code_shift);
+    }
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-        if (v + 1 < 4) {
-            W[(v + 1) & 1][0] = fetch_operand<B>(Q, j, v + 1, 0, lbase[v + 1], code_shift);
-            W[(v + 1) & 1][1] = fetch_operand<B>(Q, j, v + 1, 1, lbase[v + 1], code_shift);
+        if (v + AHEAD < 4) {
+            W[(v + AHEAD) % (AHEAD + 1)][0] =
+                fetch_operand<B, PERM>(Q, j, v + AHEAD, 0, lbase[v + AHEAD], code_shift);
+            W[(v + AHEAD) % (AHEAD + 1)][1] =
+                fetch_operand<B, PERM>(Q, j, v + AHEAD, 1, lbase[v + AHEAD], code_shift);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int d = 0; d < 2; ++d)
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
-                acc[mb][v * 2 + d] = mfma16<BF16>(W[v & 1][d], Aj[mb], acc[mb][v * 2 + d]);
+                acc[mb][v * 2 + d] =
+                    mfma16<BF16>(W[v % (AHEAD + 1)][d], Aj[mb], acc[mb][v * 2 + d]);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
 
 // B1 > 0: single stream of that width.  B1 == 0: widths read from the
 // parameters, one or two streams.
-template <int MB, int KW, int MW, bool BF16, int B1>
+template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false>
 __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int NT = 64 * KW * MW;
@@ -208,24 +233,79 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     const int wx = rho >> 3;
     const int th = wx * 32 + (rho & 7) * 4 + kg;
 
-    // ---- pair tables ------------------------------------------------------------
+    GEMM_TRACE(0);
+    const int gbeg = z * p.gper, gend = min(p.G, gbeg + p.gper);
+    const bool active = mb0 < p.mblk_total;            // whole wavefront
+    const int g0 = gbeg + kw;
+    int left = (active && g0 < gend) ? (gend - g0 + KW - 1) / KW : 0;   // tiles of this wavefront
+    const int64_t jstep = (int64_t)p.mblk_pad * 64;    // u4 units between the halves of a tile
+    // Ap is padded to whole workgroups of blocks (zeros), so every block index below
+    // gridDim.y * MW * MB is loadable.
+    const u4_t *ap = p.Ap + ((int64_t)g0 * 2 * p.mblk_pad + mb0) * 64 + lane;
+    auto load_a = [&](u4_t (&Aj)[MB], const u4_t *src) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) Aj[mb] = src[mb * 64];
+    };
+    // fast path: first tile and first activation operands are requested before the
+    // tables are built, so their latency hides behind the build
+    u4_t R[4], A0[MB], A1[MB];
+    const uint8_t *tp = p.q[0] + ((int64_t)t * p.G + g0) * 4096 + lane * 16;
+    auto load_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) R[i] = __builtin_nontemporal_load((const u4_t *)(tp + i * 1024));
+    };
     const int ngrp = p.gs >= 128 ? 1 : 128 / p.gs;
-    for (int s = 0; s < p.nstreams; ++s) {
-        const int b = B1 > 0 ? B1 : p.bits[s];
-        const int rl = p.rep_log2[s];
-        const int total = ngrp << (2 * b + rl);
-        uint32_t *tab = (uint32_t *)(smem + p.tab_off[s]);
-        const uint16_t *lut = p.lut[s];
-        for (int i = tid; i < total; i += NT) {
-            const int code = (i >> rl) & ((1 << (2 * b)) - 1);
-            const int gl = i >> (rl + 2 * b);
+    uint32_t lutv[2] = {0u, 0u};                       // fast path: LUT row(s), one value per lane
+    if constexpr (PERM) {
+#pragma unroll
+        for (int gl = 0; gl < 2; ++gl) {
+            if (gl >= ngrp) break;
             int row = p.gs >= 128 ? (t * 128) / p.gs : t * ngrp + gl;
             row = min(row, p.lut_rows - 1);
-            const uint16_t *lr = lut + ((size_t)row << b);
-            tab[i] = (uint32_t)lr[code & ((1 << b) - 1)] | ((uint32_t)lr[code >> b] << 16);
+            lutv[gl] = p.lut[0][((size_t)row << 4) + (lane & 15)];
+        }
+        if (left > 0) {
+            load_tile();
+            load_a(A0, ap);
+            load_a(A1, ap + jstep);
+        }
+    }
+
+    // ---- pair tables ------------------------------------------------------------
+    if constexpr (PERM) {
+        // 64 replicas per entry: a wavefront writes one entry per instruction, every
+        // lane the same dword, built from two lane reads of the LUT row it holds.
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+#pragma unroll
+        for (int gl = 0; gl < 2; ++gl) {
+            if (gl >= ngrp) break;
+            const uint32_t lv = lutv[gl];
+            uint32_t *tab = (uint32_t *)(smem + p.tab_off[0]) + (gl << 14);
+            for (int code = wave_u; code < 256; code += NT / 64) {
+                const uint32_t lo = __builtin_amdgcn_readlane(lv, code & 15);
+                const uint32_t hi = __builtin_amdgcn_readlane(lv, code >> 4);
+                tab[code * 64 + lane] = lo | (hi << 16);
+            }
+        }
+    } else {
+        for (int s = 0; s < p.nstreams; ++s) {
+            const int b = B1 > 0 ? B1 : p.bits[s];
+            const int rl = p.rep_log2[s];
+            const int total = ngrp << (2 * b + rl);
+            uint32_t *tab = (uint32_t *)(smem + p.tab_off[s]);
+            const uint16_t *lut = p.lut[s];
+            for (int i = tid; i < total; i += NT) {
+                const int code = (i >> rl) & ((1 << (2 * b)) - 1);
+                const int gl = i >> (rl + 2 * b);
+                int row = p.gs >= 128 ? (t * 128) / p.gs : t * ngrp + gl;
+                row = min(row, p.lut_rows - 1);
+                const uint16_t *lr = lut + ((size_t)row << b);
+                tab[i] = (uint32_t)lr[code & ((1 << b) - 1)] | ((uint32_t)lr[code >> b] << 16);
+            }
         }
     }
     __syncthreads();
+    GEMM_TRACE(1);
 
     f4_t acc[MB][8];
 #pragma unroll
@@ -233,18 +313,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[mb][i] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const int gbeg = z * p.gper, gend = min(p.G, gbeg + p.gper);
-    const bool active = mb0 < p.mblk_total;            // whole wavefront
-    // Operand blocks past the padded M alias block 0; their sums are never stored.
-    int mbi[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) mbi[mb] = (mb0 + mb < p.mblk_total) ? mb0 + mb : 0;
-
-    auto load_a = [&](u4_t (&Aj)[MB], int g, int j) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            Aj[mb] = p.Ap[(((int64_t)g * 2 + j) * p.mblk_total + mbi[mb]) * 64 + lane];
-    };
     const uint32_t lds_base =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     auto table_bases = [&](uint32_t (&lb)[4], int s, int b) {
@@ -259,38 +327,108 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     };
 
     if (active) {
-        if constexpr (B1 > 0) {
+        if constexpr (PERM) {
+            // 4-bit fast path.  A 64-byte chunk per lane is the worst pattern for the
+            // vector memory pipe (one 64-byte sector per lane and instruction), so the
+            // 4 KB tile is fetched as four fully contiguous 1 KB rows instead, dropped
+            // into a per-wavefront LDS buffer and read back chunk by chunk.  Slot
+            // order and a rotation of the four quarters keep both sides free of bank
+            // conflicts: piece (chunk c, quarter kt) lives at
+            //     (c ^ ((c >> 4) & 1)) * 64 + ((kt + (c >> 2)) & 3) * 16.
+            typedef __attribute__((address_space(3))) u4_t *LdsQuad;
+            uint32_t lb[4];
+            table_bases(lb, 0, 4);
+            const uint32_t stage = lds_base + p.stage_off + wave * 4096;
+            const int rotw = ((lane & 3) + ((lane >> 4) & 3)) & 3;
+            const uint32_t wb_even = stage + (lane >> 2) * 64 + rotw * 16;
+            const uint32_t wb_odd = stage + ((lane >> 2) ^ 1) * 64 + rotw * 16;
+            const int slot = th ^ ((th >> 4) & 1);
+            uint32_t rb[4];
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) rb[kt] = stage + slot * 64 + ((kt + (rho & 3)) & 3) * 16;
+
+            uint32_t Q[16];
+            constexpr int64_t qstep = (int64_t)KW * 4096;
+            const int64_t astep = (int64_t)KW * 2 * p.mblk_pad * 64;
+            auto stage_write = [&]() {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    *(LdsQuad)(uintptr_t)(((i & 1) ? wb_odd : wb_even) + i * 1024) = R[i];
+            };
+            auto stage_read = [&]() {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) {
+                    const u4_t v = *(LdsQuad)(uintptr_t)rb[kt];
+                    Q[4 * kt + 0] = v[0];
+                    Q[4 * kt + 1] = v[1];
+                    Q[4 * kt + 2] = v[2];
+                    Q[4 * kt + 3] = v[3];
+                }
+            };
+            if (left > 0) {
+                stage_write();                            // first tile, requested before the tables
+                if (left > 1) tp += qstep;
+                load_tile();                              // second tile (or a harmless reload)
+            }
+            int it = 0;
+            while (left > 0) {
+                stage_read();                             // this tile's chunk
+                __builtin_amdgcn_sched_barrier(0);
+                half_mma<4, MB, BF16, true>(Q, 0, A0, acc, lb, 8);
+                if (left > 1) ap += astep;
+                load_a(A0, ap);                           // half a tile ahead of its use
+                stage_write();                            // next tile, requested a whole tile ago
+                if (left > 2) tp += qstep;
+                load_tile();                              // the tile after it
+                __builtin_amdgcn_sched_barrier(0);
+                half_mma<4, MB, BF16, true>(Q, 1, A1, acc, lb, 8);
+                load_a(A1, ap + jstep);
+                __builtin_amdgcn_sched_barrier(0);
+                if (it < 10) GEMM_TRACE(6 + it);
+                ++it;
+                --left;
+            }
+        } else if constexpr (B1 > 0) {
             uint32_t lb[4];
             table_bases(lb, 0, B1);
             const int cs = p.rep_log2[0] + 2;
-            uint32_t Qc[4 * B1], Qn[4 * B1];
-            u4_t A0[MB], A1[MB];
-            int g = gbeg + kw;
-            if (g < gend) {
-                load_chunk<B1>(Qc, p.q[0], (int64_t)t * p.G + g, th);
-                load_a(A0, g, 0);
-                load_a(A1, g, 1);
+            uint32_t Qa[4 * B1], Qb[4 * B1];
+            const uint8_t *qp = p.q[0] + (((int64_t)t * p.G + g0) * 64 + th) * (16 * B1);
+            constexpr int64_t qstep = (int64_t)KW * 64 * 16 * B1;
+            const int64_t astep = (int64_t)KW * 2 * p.mblk_pad * 64;
+            if (left > 0) {
+                load_chunk<B1>(Qa, qp);
+                load_a(A0, ap);
+                load_a(A1, ap + jstep);
             }
-            while (g < gend) {
-                const int gn = g + KW;
-                const int gl = gn < gend ? gn : g;      // harmless reload on the last pass
-                load_chunk<B1>(Qn, p.q[0], (int64_t)t * p.G + ((p.dbg & 1) ? gbeg : gl), th);
+            // One tile: the next chunk is requested first (a whole tile ahead), the
+            // activation halves of the next tile as soon as their registers are free.
+            auto step = [&](const uint32_t (&Qc)[4 * B1], uint32_t (&Qn)[4 * B1], bool more) {
+                if (more) {                              // else: harmless reload of this tile
+                    qp += qstep;
+                    ap += astep;
+                }
+                load_chunk<B1>(Qn, qp);
                 __builtin_amdgcn_sched_barrier(0);
-                half_mma<B1, MB, BF16>(Qc, 0, A0, acc, lb, cs);
-                load_a(A0, (p.dbg & 2) ? gbeg : gl, 0);  // half a tile ahead of its use
+                half_mma<B1, MB, BF16, PERM>(Qc, 0, A0, acc, lb, cs);
+                load_a(A0, ap);
                 __builtin_amdgcn_sched_barrier(0);
-                half_mma<B1, MB, BF16>(Qc, 1, A1, acc, lb, cs);
-                load_a(A1, (p.dbg & 2) ? gbeg : gl, 1);
+                half_mma<B1, MB, BF16, PERM>(Qc, 1, A1, acc, lb, cs);
+                load_a(A1, ap + jstep);
                 __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int i = 0; i < 4 * B1; ++i) Qc[i] = Qn[i];
-                g = gn;
+            };
+            while (left > 0) {
+                step(Qa, Qb, left > 1);
+                if (--left == 0) break;
+                step(Qb, Qa, left > 1);
+                --left;
             }
         } else {
             for (int g = gbeg + kw; g < gend; g += KW) {
                 u4_t A0[MB], A1[MB];
-                load_a(A0, g, 0);
-                load_a(A1, g, 1);
+                const u4_t *ap = p.Ap + ((int64_t)g * 2 * p.mblk_pad + mb0) * 64 + lane;
+                load_a(A0, ap);
+                load_a(A1, ap + jstep);
                 for (int s = 0; s < p.nstreams; ++s) {
                     uint32_t lb[4];
                     const int cs = p.rep_log2[s] + 2;
@@ -299,28 +437,28 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                         case 1: {
                             uint32_t Q[4];
                             table_bases(lb, s, 1);
-                            load_chunk<1>(Q, p.q[s], tile, th);
+                            load_chunk<1>(Q, p.q[s] + (tile * 64 + th) * (16 * 1));
                             half_mma<1, MB, BF16>(Q, 0, A0, acc, lb, cs);
                             half_mma<1, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
                         case 2: {
                             uint32_t Q[8];
                             table_bases(lb, s, 2);
-                            load_chunk<2>(Q, p.q[s], tile, th);
+                            load_chunk<2>(Q, p.q[s] + (tile * 64 + th) * (16 * 2));
                             half_mma<2, MB, BF16>(Q, 0, A0, acc, lb, cs);
                             half_mma<2, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
                         case 3: {
                             uint32_t Q[12];
                             table_bases(lb, s, 3);
-                            load_chunk<3>(Q, p.q[s], tile, th);
+                            load_chunk<3>(Q, p.q[s] + (tile * 64 + th) * (16 * 3));
                             half_mma<3, MB, BF16>(Q, 0, A0, acc, lb, cs);
                             half_mma<3, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
                         default: {
                             uint32_t Q[16];
                             table_bases(lb, s, 4);
-                            load_chunk<4>(Q, p.q[s], tile, th);
+                            load_chunk<4>(Q, p.q[s] + (tile * 64 + th) * (16 * 4));
                             half_mma<4, MB, BF16>(Q, 0, A0, acc, lb, cs);
                             half_mma<4, MB, BF16>(Q, 1, A1, acc, lb, cs);
                         } break;
@@ -332,7 +470,9 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 
     // ---- tree over the KW wavefronts of one m group, through LDS ------------------
     f4_t *red = (f4_t *)smem;                           // slot = [MB*8][64] f4
+    GEMM_TRACE(2);
     __syncthreads();                                    // tables are dead from here
+    GEMM_TRACE(3);
 #pragma unroll
     for (int step = KW / 2; step >= 1; step >>= 1) {
         if (kw >= step && kw < 2 * step) {
@@ -353,22 +493,42 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         __syncthreads();
     }
 
-    // ---- across workgroups: partial images + ticket --------------------------------
+    GEMM_TRACE(4);
+    // ---- totals of the workgroup as a row-major fp32 tile in LDS --------------------
+    constexpr int ROWS = MW * MB * 16;                  // rows of C this workgroup owns
+    constexpr int LDT = 128 + 4;                        // padded row: conflict-free both ways
+    float *tile = (float *)smem;
+    if (kw == 0) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int row = (mw * MB + mb) * 16 + rho;
+                const int n0 = (kg >> 1) * 64 + (i >> 1) * 16 + (i & 1) * 8 + (kg & 1) * 4;
+                *(f4_t *)(tile + row * LDT + n0) = acc[mb][i];
+            }
+    }
+    __syncthreads();
+
+    // Every thread now serves pieces of 8 consecutive outputs of one row: 16 threads
+    // write one 256-byte row segment of C.
+    constexpr int PIECES = ROWS * 16;
+    const int unit = blockIdx.y * gridDim.x + blockIdx.x;           // (m chunk, n tile)
+    const size_t image = (size_t)ROWS * 128;                        // floats per unit per z
+    const size_t zstride = (size_t)gridDim.x * gridDim.y * image;
     if (p.ksplit > 1) {
-        const int unit = blockIdx.y * gridDim.x + blockIdx.x;       // (m chunk, n tile)
-        const size_t image = (size_t)MW * MB * 8 * 64 * 4;          // floats per unit per z
-        float *mine = p.P + ((size_t)z * gridDim.x * gridDim.y + unit) * image;
-        if (kw == 0) {
+        // across workgroups: partial tiles + ticket; the last arrival folds them in z order
+        float *mine = p.P + (size_t)z * zstride + (size_t)unit * image;
+        for (int idx = tid; idx < PIECES; idx += NT) {
+            const int ml = idx >> 4, n8 = idx & 15;
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    gemm_ws_store(mine + ((size_t)(mw * MB + mb) * 8 + i) * 256 + lane * 4,
-                                  acc[mb][i]);
+            for (int e = 0; e < 8; ++e)
+                __hip_atomic_store(mine + ml * 128 + n8 * 8 + e, tile[ml * LDT + n8 * 8 + e],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
-        int *flag = (int *)smem;
+        int *flag = (int *)(tile + ROWS * LDT);
         if (tid == 0) {
             const int old = __hip_atomic_fetch_add(p.tickets + unit, 1, __ATOMIC_RELAXED,
                                                    __HIP_MEMORY_SCOPE_AGENT);
@@ -376,76 +536,73 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         }
         __syncthreads();
         if (!*flag) return;
-        if (kw == 0) {
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    f4_t s = {0.0f, 0.0f, 0.0f, 0.0f};
-                    const float *src = p.P + (size_t)unit * image +
-                                       ((size_t)(mw * MB + mb) * 8 + i) * 256 + lane * 4;
-                    const size_t zstride = (size_t)gridDim.x * gridDim.y * image;
-                    for (int z0 = 0; z0 < p.ksplit; z0 += 4) {     // 16 loads in flight
-                        float part[4][4];
-#pragma unroll
-                        for (int a = 0; a < 4; ++a)
-#pragma unroll
-                            for (int r = 0; r < 4; ++r)
-                                part[a][r] = (z0 + a < p.ksplit)
-                                                 ? gemm_ws_load(src + (z0 + a) * zstride + r)
-                                                 : 0.0f;
-#pragma unroll
-                        for (int a = 0; a < 4; ++a)
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) s[r] += part[a][r];
-                    }
-                    acc[mb][i] = s;
-                }
-        }
         if (tid == 0)
             __hip_atomic_store(p.tickets + unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- epilogue: residual, bias, one rounding, store -------------------------------
-    if (kw != 0 || !active) return;
-    const int nb = t * 128 + (kg >> 1) * 64 + (kg & 1) * 4;
+    for (int idx = tid; idx < PIECES; idx += NT) {
+        const int ml = idx >> 4, n8 = idx & 15;
+        const int m = blockIdx.y * ROWS + ml;
+        if (m >= p.M) continue;
+        const int n0 = t * 128 + n8 * 8;
+        float y[8];
+        if (p.ksplit > 1) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int m = (mb0 + mb) * 16 + rho;
-        if (mb0 + mb >= p.mblk_total || m >= p.M) continue;
+            for (int e = 0; e < 8; ++e) y[e] = 0.0f;
+            const float *src = p.P + (size_t)unit * image + ml * 128 + n8 * 8;
+            for (int z0 = 0; z0 < p.ksplit; z0 += 2) {         // 16 loads in flight
+                float part[2][8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int n0 = nb + (i >> 1) * 16 + (i & 1) * 8;
-            f4_t y = acc[mb][i];
-            if (p.R > 0) {
-                const float *xr = p.xb + (size_t)m * p.R;
-                for (int r = 0; r < p.R; ++r) {
-                    const float c = xr[r];
+                for (int a = 0; a < 2; ++a)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        y[e] = fmaf(c, load_act(p.resA, (int64_t)(n0 + e) * p.R + r, p.out_bf16),
-                                    y[e]);
-                }
+                    for (int e = 0; e < 8; ++e)
+                        part[a][e] = (z0 + a < p.ksplit) ? gemm_ws_load(src + (z0 + a) * zstride + e)
+                                                         : 0.0f;
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) y[e] += part[a][e];
             }
-            if (p.bias) {
+        } else {
+            const f4_t lo = *(const f4_t *)(tile + ml * LDT + n8 * 8);
+            const f4_t hi = *(const f4_t *)(tile + ml * LDT + n8 * 8 + 4);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) y[e] += load_act(p.bias, n0 + e, p.out_bf16);
+            for (int e = 0; e < 4; ++e) {
+                y[e] = lo[e];
+                y[4 + e] = hi[e];
             }
-            uint16_t o[4];
+        }
+        if (p.R > 0) {
+            const float *xr = p.xb + (size_t)m * p.R;
+            for (int r = 0; r < p.R; ++r) {
+                const float c = xr[r];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = round_act(y[e], p.out_bf16);
-            uint16_t *dst = (uint16_t *)p.C + (size_t)m * p.ldc + n0;
-            if (p.vec_store) {
-                uint2 pk;
-                pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-                pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-                *(uint2 *)dst = pk;
-            } else {
+                for (int e = 0; e < 8; ++e)
+                    y[e] = fmaf(c, load_act(p.resA, (int64_t)(n0 + e) * p.R + r, p.out_bf16), y[e]);
+            }
+        }
+        if (p.bias) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) dst[e] = o[e];
+            for (int e = 0; e < 8; ++e) y[e] += load_act(p.bias, n0 + e, p.out_bf16);
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            o[e] = (uint32_t)round_act(y[2 * e], p.out_bf16) |
+                   ((uint32_t)round_act(y[2 * e + 1], p.out_bf16) << 16);
+        uint16_t *dst = (uint16_t *)p.C + (size_t)m * p.ldc + n0;
+        if (p.vec_store) {
+            *(u4_t *)dst = u4_t{o[0], o[1], o[2], o[3]};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                dst[2 * e] = (uint16_t)o[e];
+                dst[2 * e + 1] = (uint16_t)(o[e] >> 16);
             }
         }
     }
+    GEMM_TRACE(5);
 }
 
 }  // namespace flute
