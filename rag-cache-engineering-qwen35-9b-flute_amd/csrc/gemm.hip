@@ -15,11 +15,14 @@ struct GemmShape {
 };
 
 // M <= 16: one block, eight k ways (the launch is a weight stream, like the GEMV).
-// M <= 64: four blocks, eight k ways.  Larger: 128 rows of A per workgroup, two m
-// groups of four blocks, four k ways; further rows go to gridDim.y.
-GemmShape choose_gemm_shape(int M) {
-    if (M <= 16) return {1, 8, 1, 2};
-    if (M <= 64) return {4, 8, 1, 1};
+// Otherwise four blocks per wavefront: 64 rows of A per workgroup with eight k ways
+// while that still fits the device in one round of workgroups, else 128 rows (two m
+// groups, four k ways); further rows go to gridDim.y.  The tables plus staging take
+// most of a CU's LDS, so one workgroup per CU is resident.
+GemmShape choose_gemm_shape(int M, int tiles) {
+    if (M <= 16) return {1, 8, 1, 1};
+    const int chunks64 = (M + 63) / 64;
+    if ((int64_t)tiles * chunks64 <= kNumCU) return {4, 8, 1, 1};
     return {4, 4, 2, 1};
 }
 
@@ -43,8 +46,11 @@ flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t st
 template <bool BF16>
 flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 grid, int lds,
                                hipStream_t stream) {
-    if (!BF16 && s.mw == 2 && p.nstreams == 1 && p.bits[0] == 4 && p.rep_log2[0] == 6)
+    if (!BF16 && p.nstreams == 1 && p.bits[0] == 4 && p.rep_log2[0] == 6) {
+        if (s.mb == 1) return launch_gemm<1, 8, 1, false, 4, true>(p, grid, lds, stream);
+        if (s.mw == 1) return launch_gemm<4, 8, 1, false, 4, true>(p, grid, lds, stream);
         return launch_gemm<4, 4, 2, false, 4, true>(p, grid, lds, stream);
+    }
     set_error("flute_gemm: development build without this kernel");
     return FLUTE_ERR_UNSUPPORTED;
 }
@@ -101,7 +107,7 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
                   M, w->R);
     hipStream_t stream = (hipStream_t)stream_;
 
-    GemmShape shape = choose_gemm_shape(M);
+    GemmShape shape = choose_gemm_shape(M, w->N / 128);
     GemmParams p = {};
     p.nstreams = w->b2 > 0 ? 2 : 1;
     p.q[0] = (const uint8_t *)w->q1;

@@ -111,8 +111,25 @@ __global__ void __launch_bounds__(256) gemm_coeff_kernel(const uint16_t *A, int6
     if (threadIdx.x == 0) xb[(int64_t)m * R + r] = red[0];
 }
 
-__device__ __forceinline__ float gemm_ws_load(const float *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Partial sums cross workgroups (and so the per-XCD L2s) inside one launch: they are
+// written through and read around the L2 with device-scope (sc1) accesses, the same
+// instructions a relaxed agent-scope atomic compiles to, but 16 bytes at a time.
+__device__ __forceinline__ void ws_store16(float *p, f4_t v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void ws_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Four 16-byte device-scope loads in flight, complete on return.
+__device__ __forceinline__ void ws_load16x4(const float *p0, const float *p1, const float *p2,
+                                            const float *p3, f4_t &a, f4_t &b, f4_t &c, f4_t &d) {
+    asm volatile(
+        "global_load_dwordx4 %0, %4, off sc1\n"
+        "global_load_dwordx4 %1, %5, off sc1\n"
+        "global_load_dwordx4 %2, %6, off sc1\n"
+        "global_load_dwordx4 %3, %7, off sc1\n"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d)
+        : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+        : "memory");
 }
 
 #ifdef FLUTE_GEMM_TRACE
@@ -521,11 +538,10 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         float *mine = p.P + (size_t)z * zstride + (size_t)unit * image;
         for (int idx = tid; idx < PIECES; idx += NT) {
             const int ml = idx >> 4, n8 = idx & 15;
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                __hip_atomic_store(mine + ml * 128 + n8 * 8 + e, tile[ml * LDT + n8 * 8 + e],
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ws_store16(mine + ml * 128 + n8 * 8, *(const f4_t *)(tile + ml * LDT + n8 * 8));
+            ws_store16(mine + ml * 128 + n8 * 8 + 4, *(const f4_t *)(tile + ml * LDT + n8 * 8 + 4));
         }
+        ws_stores_done();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         int *flag = (int *)(tile + ROWS * LDT);
@@ -551,18 +567,23 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 #pragma unroll
             for (int e = 0; e < 8; ++e) y[e] = 0.0f;
             const float *src = p.P + (size_t)unit * image + ml * 128 + n8 * 8;
-            for (int z0 = 0; z0 < p.ksplit; z0 += 2) {         // 16 loads in flight
-                float part[2][8];
+            for (int z0 = 0; z0 < p.ksplit; z0 += 2) {
+                const float *s0 = src + z0 * zstride;
+                const float *s1 = z0 + 1 < p.ksplit ? s0 + zstride : s0;
+                f4_t a, b, c, d;
+                ws_load16x4(s0, s0 + 4, s1, s1 + 4, a, b, c, d);
 #pragma unroll
-                for (int a = 0; a < 2; ++a)
+                for (int e = 0; e < 4; ++e) {
+                    y[e] += a[e];
+                    y[4 + e] += b[e];
+                }
+                if (z0 + 1 < p.ksplit) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        part[a][e] = (z0 + a < p.ksplit) ? gemm_ws_load(src + (z0 + a) * zstride + e)
-                                                         : 0.0f;
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) y[e] += part[a][e];
+                    for (int e = 0; e < 4; ++e) {
+                        y[e] += c[e];
+                        y[4 + e] += d[e];
+                    }
+                }
             }
         } else {
             const f4_t lo = *(const f4_t *)(tile + ml * LDT + n8 * 8);
