@@ -100,6 +100,58 @@ def _cpu_baseline(torch, seconds_budget=20.0):
                       f"os.cpu_count={os.cpu_count()}"}
 
 
+def _gemm_section(torch, _lib, ctypes, sets, gen, dev, O):
+    """The second half of the metric: C[M, 12288] = A[M, 4096] @ W^T on the same idx4
+    blobs (the gate projections of the weight sets), bf16 LUT, bf16 activations, bf16
+    MFMA with fp32 accumulate.  One call = flute_gemm as a caller sees it, including its
+    activation pre-pass.  Headline M = 256; the other M of the configuration are listed."""
+    lut_bf = [(torch.randn(I // GS, 16, device=dev, generator=gen) * 0.02).sort(dim=1).values
+              .to(torch.bfloat16).contiguous() for _ in sets]
+    descs = []
+    for s, lut in zip(sets, lut_bf):
+        blob = s["t"][0][0]
+        descs.append(_desc(_lib, blob, lut, I, H))
+    res = {}
+    for M in (256, 16, 64, 1024):
+        A = torch.randn(M, H, device=dev, generator=gen).to(torch.bfloat16)
+        C = torch.empty(M, I, dtype=torch.bfloat16, device=dev)
+
+        def call(i):
+            st = _lib.lib.flute_gemm(ctypes.byref(descs[i % len(descs)]), A.data_ptr(), C.data_ptr(),
+                                     M, H, I, _lib.BF16, torch.cuda.current_stream().cuda_stream)
+            if st != 0:
+                raise RuntimeError(_lib.last_error())
+
+        call(0)
+        torch.cuda.synchronize()
+        # parity against the oracle's dequantised rows of three tiles, fp64 matmul
+        blob, lut = sets[0]["t"][0][0], lut_bf[0]
+        per = (H // 64) * 4096
+        num = den = 0.0
+        Ad = A.cpu().double()
+        for tile in (0, 41, 95):
+            Wt = O.dequant(blob[tile * per:(tile + 1) * per].cpu().numpy(), lut[tile:tile + 1].cpu(),
+                           128, H, GS, 4).double()
+            ref = Ad @ Wt.t()
+            got = C[:, tile * 128:(tile + 1) * 128].cpu().double()
+            num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
+        err = (num / den) ** 0.5
+        if err > 4e-3:                      # bf16 output: rounding alone is 2^-9
+            raise SystemExit(f"bench.py: GEMM parity gate failed at M={M} ({err:.2e})")
+        n = 48
+        us = _time_graph(torch, lambda: [call(i) for i in range(n)]) / n * 1e3
+        tf = 2.0 * M * I * H / us / 1e6
+        res[M] = {"us_per_call": round(us, 2), "tflops": round(tf, 1),
+                  "frac_mfma": round(tf / MFMA_PEAK_TFLOPS, 4), "parity_rel_l2": err}
+    head = res[256]
+    return {"workload": "LUT-GEMM M=256: 4096->12288, idx4, group 128, bf16 LUT, bf16 activations, "
+                        "bf16 MFMA fp32 accumulate; whole flute_gemm call (activation pre-pass + kernel)",
+            "value": head["tflops"], "unit": "TFLOP/s", "peak": MFMA_PEAK_TFLOPS,
+            "frac": head["frac_mfma"], "us_per_call": head["us_per_call"],
+            "parity_rel_l2": head["parity_rel_l2"],
+            "other_M": {str(m): res[m] for m in (16, 64, 1024)}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,6 +159,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=24)
     ap.add_argument("--sets", type=int, default=12, help="distinct weight sets (72 MiB each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the M>1 LUT-GEMM section")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N "
@@ -203,6 +256,8 @@ def main():
     value = bytes_step / (ms_step * 1e-3) / 1e9
     achieved = bytes_gate_up / (ms_gu * 1e-3) / 1e9
 
+    gemm = None if args.no_gemm else _gemm_section(torch, _lib, ctypes, sets, gen, dev, O)
+
     out = {
         "metric": "M=1 LUT-GEMV achieved HBM GB/s (% of peak); M=256 LUT-GEMM TFLOP/s (% MFMA)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -221,6 +276,8 @@ def main():
                      "us_per_launch": round(ms_gu * 1e3, 3),
                      "algorithmic_bytes_per_launch": bytes_gate_up},
     }
+    if gemm is not None:
+        out["gemm"] = gemm
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = _cpu_baseline(torch)
     print(json.dumps(out))
