@@ -139,6 +139,9 @@ flute_status flute_mlp_block(const flute_linear *gate, const flute_linear *up,
  * (src/bindings.cpp:257-270).  The MFMA operand type follows lut_dtype, so the
  * dequantised tile is exactly the LUT entry; A is converted to that type if it
  * differs.  lda = row stride of A in elements (>= K), ldc likewise for C.
+ * When w->signs is set the rows of A are rotated first (a flute_fht pass into the
+ * library workspace), as the M = 1 entry does in its prologue.  The fused residual
+ * serves M * R <= 16384; larger products are refused with FLUTE_ERR_UNSUPPORTED.
  */
 flute_status flute_gemm(const flute_linear *w, const void *A, void *C, int M,
                         int64_t lda, int64_t ldc, int act_dtype, void *stream);

@@ -185,9 +185,10 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     const size_t p_floats = ksplit > 1 ? (size_t)ksplit * units * image : 0;
     const size_t xb_floats = ((size_t)M * w->R + 3) & ~(size_t)3;
     const size_t ap_floats = (size_t)p.G * 2 * p.mblk_pad * 64 * 4;
+    const size_t rot_floats = w->signs ? ((size_t)M * w->K / 2 + 4) & ~(size_t)3 : 0;
     float *base = nullptr;
     int *tickets = nullptr;
-    st = get_workspace(p_floats + xb_floats + ap_floats + 64, (size_t)units + 1, stream, &base,
+    st = get_workspace(p_floats + xb_floats + ap_floats + rot_floats + 64, (size_t)units + 1, stream, &base,
                        &tickets);
     if (st != FLUTE_OK) return st;
     p.P = base;
@@ -195,6 +196,15 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     float *xb = base + p_floats;
     u4_t *Ap = (u4_t *)(xb + xb_floats);
     p.Ap = Ap;
+    if (w->signs) {
+        // rotated copy of the activations (the transform needs whole rows), then the
+        // ordinary pre-pass on it
+        void *Arot = (void *)(Ap + (size_t)p.G * 2 * p.mblk_pad * 64);
+        st = flute_fht(A, w->signs, w->awq, Arot, M, w->K, act_dtype, 0, w->rot_block, stream_);
+        if (st != FLUTE_OK) return st;
+        A = Arot;
+        lda = w->K;
+    }
 
     {
         const int64_t total = (int64_t)p.G * 2 * p.mblk_pad * 64;

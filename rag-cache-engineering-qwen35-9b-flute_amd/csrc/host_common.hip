@@ -69,13 +69,10 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who) {
     FLUTE_REQUIRE(w->awq == nullptr || w->signs != nullptr, FLUTE_ERR_INVALID,
                   "%s: awq scale only exists as a companion to the rotation signs", who);
     if (w->signs != nullptr) {
-        FLUTE_REQUIRE(mode == 0, FLUTE_ERR_UNSUPPORTED,
-                      "%s: the fused rotation is a GEMV prologue; rotate the GEMM input with "
-                      "flute_fht first",
-                      who);
         FLUTE_REQUIRE(w->K % 32 == 0 && w->K >= 32 && w->K <= 65504, FLUTE_ERR_INVALID,
                       "%s: rotation needs K %% 32 == 0 and 32 <= K <= 65504 (got %d)", who, w->K);
-        const Segs sg = make_segments(w->K, 0);
+        (void)mode;
+        const Segs sg = make_segments(w->K, w->rot_block);
         FLUTE_REQUIRE(sg.len[0] <= 16384, FLUTE_ERR_UNSUPPORTED,
                       "%s: rotation segment %d exceeds 16384 columns", who, sg.len[0]);
     }

@@ -152,3 +152,48 @@ def test_fused_mlp_module():
     y = mker(x.to(DEV))
     assert pm.ROUTE_CENSUS.get("gemv_mlp") == 1 and mker._merge_state["ok"]
     assert rel_l2(y.cpu(), mref(x)) <= 2e-3       # two 16-bit roundings (h, then y) on each side
+
+
+@pytest.mark.parametrize("M,spec,route", [
+    (8, dict(), "dual_stream"),
+    (16, dict(bits2=2, rank=8, bias=True), "dual_stream"),
+    (40, dict(bits2=2, rank=8, bias=True), "per_group_lut"),
+    (130, dict(bits=3, gs=32), "per_group_lut"),
+])
+@pytest.mark.parametrize("rot", [False, True])
+def test_module_kernel_mode_matches_reference_mode_prefill(M, spec, route, rot):
+    """M > 1 goes to the MFMA GEMM: the fused small-M entry up to 16 rows, the plain
+    entry (second stream, residual and bias added by the module) above."""
+    N, K = 512, 1024
+    w = make_weight(N, K, seed=5, **spec)
+    kw = dict(rotation_seed=9, rotation_k=K) if rot else {}
+    ref, ker = _modules(w, **kw)
+    x = make_x(M, K, seed=6)
+    pm.ROUTE_CENSUS.clear()
+    y = ker(x.to(DEV))
+    assert y.shape == (M, N)
+    assert rel_l2(y.cpu(), ref(x)) <= (TOL if M <= 16 else 2e-3)   # module-side adds round twice
+    assert list(pm.ROUTE_CENSUS) == [route]
+
+
+def test_gemm_with_rotation_through_the_c_abi():
+    """flute_gemm rotates its input itself when the descriptor carries signs
+    (block-128 form and the full-K form), M = 8 as in the rotated-input configuration."""
+    N, K, M = 512, 4096, 8
+    w = make_weight(N, K, seed=11, device=DEV)
+    x = make_x(M, K, seed=12, dtype=torch.bfloat16)
+    xd = x.to(DEV)
+    for block in (128, 0):
+        signs = O.rotation_signs(K, 3)
+        sd = signs.to(DEV)
+        d = _desc(w)
+        d.signs, d.rot_block = sd.data_ptr(), block
+        C = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+        st = _lib.lib.flute_gemm(ctypes.byref(d), xd.data_ptr(), C.data_ptr(), M, K, N, _lib.BF16,
+                                 torch.cuda.current_stream().cuda_stream)
+        assert st == 0, _lib.last_error()
+        xr = O.block_fht_reference(x, 128, signs) if block else O.fht_reference(x, signs)
+        # the rotated activations are rounded to bf16 before the GEMM, then cast to the
+        # LUT's fp16 (exact for these magnitudes)
+        ref = _exact(w, xr.to(torch.bfloat16).half()).to(torch.bfloat16)
+        assert rel_l2(C.cpu(), ref) <= 4e-3
