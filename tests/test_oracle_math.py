@@ -3,6 +3,7 @@ forward, SiLU*mul, the rotation and the split policy, each against something
 the mathematics fixes rather than against its own formula."""
 import ctypes
 import math
+import json
 import os
 
 import numpy as np
@@ -144,15 +145,35 @@ def test_block_fht_and_awq():
     assert np.abs(O.fht_awq_reference(x, signs, s).double().numpy() - exp).max() < 1e-4
 
 
+def _golden():
+    with open(os.path.join(ROOT, "tests", "golden", "reference_stated_examples.json")) as f:
+        return json.load(f)
+
+
 def test_upstream_split_policy_examples():
-    """(tiles, K) -> split, the worked examples of src/kernel_gemv_splitk.cu:54-59."""
-    cases = [(4, 4096, 16), (8, 4096, 16), (16, 4096, 16), (32, 4096, 8), (32, 12288, 8),
-             (64, 4096, 4), (96, 4096, 2), (1940, 4096, 1)]
+    """(tiles, K) -> split and workgroup count: the worked examples upstream states in
+    src/kernel_gemv_splitk.cu:54-59, held as data in tests/golden."""
     lib = None
     path = os.path.join(ROOT, "oracle", "liboracle.so")
     if os.path.exists(path):
         lib = ctypes.CDLL(path)
-    for tiles, K, want in cases:
+    cases = _golden()["split_policy"]["cases"]
+    assert len(cases) >= 7
+    for tiles, K, want, wgs in cases:
         assert O.pick_split_upstream(tiles, K // 64) == want
+        assert tiles * want == wgs
         if lib is not None:
             assert lib.oracle_pick_split_upstream(tiles, K // 64) == want
+
+
+def test_upstream_segment_examples():
+    """The decompositions upstream lists in the docstring of segments (fht.py:118-124)."""
+    for K, want in _golden()["segments"]["cases"].items():
+        assert O.segments(int(K)) == [tuple(p) for p in want]
+        assert sum(b for _, b in O.segments(int(K))) == int(K)
+
+
+def test_blob_geometry_constants():
+    g = _golden()["blob_geometry"]
+    assert (O.ROWS_PER_TILE, O.K_PER_TILE, O.CHUNKS_PER_TILE, O.PAIRS_PER_CHUNK) == \
+        (g["tile_rows"], g["tile_k"], g["chunks_per_tile"], g["pairs_per_chunk"])
