@@ -30,6 +30,10 @@ sys.path[:0] = [os.path.join(ROOT, "rag-cache-engineering-qwen35-9b-flute_amd")]
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X published dense bf16/fp16 MFMA rate
 H, I, GS = 4096, 12288, 128
+# HBM bytes one launch of the merged gate+up kernel moves, from FETCH_SIZE and WRITE_SIZE
+# counter runs of this file scaled by a copy of known size (--calibrate-copy); the readings
+# are kept in profiles/gemv4_gate_up_hbm_traffic.txt.  Only valid for the default workload.
+TRAFFIC_GATE_UP_BYTES = 50729650
 
 
 def _weights(torch, N, K, gen, dev, lut_dtype):
@@ -160,6 +164,9 @@ def main():
     ap.add_argument("--sets", type=int, default=12, help="distinct weight sets (72 MiB each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M>1 LUT-GEMM section")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 64 MiB device copy, so that a counter run of this "
+                         "command holds a kernel of known traffic to scale FETCH_SIZE/WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N "
@@ -238,6 +245,12 @@ def main():
         print(f"bench.py: parity gate failed (h {err_h:.2e}, y {err_y:.2e})", file=sys.stderr)
         return 1
 
+    if args.calibrate_copy:
+        src = torch.randint(0, 255, (64 << 20,), dtype=torch.uint8, device=dev, generator=gen)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+
     # ---- timed region 1: whole MLP blocks ------------------------------------------
     for i in range(args.warmup):
         block(sets[i % args.sets])
@@ -271,7 +284,7 @@ def main():
                    "timing": "hipGraph replay, events on the launch stream",
                    "parity_rel_l2": {"h": err_h, "y": err_y}},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_GATE_UP_BYTES,
                      "kernel": "gemv4_kernel (merged gate+up, SiLU*mul)",
                      "us_per_launch": round(ms_gu * 1e3, 3),
                      "algorithmic_bytes_per_launch": bytes_gate_up},
