@@ -1,0 +1,244 @@
+"""Reader of palettized weight artifacts: one metadata record + the raw member
+files of an artifact directory -> a PalettizedLinear or a SplitQKV.
+
+Mirrors the upstream reader (src/scripts/palettized_modules.py:229-330 for the
+name/layout rules, :2411-2483 `_read_indices_and_lut`, :2486-2500 `_read_residual`,
+:2503-2590 `_read_stream2`, :2619-2724 `load_palettized_weight`): same metadata
+keys, same validation order, same exceptions (ValueError naming the tensor and
+the fix).  Member files are raw little-endian arrays without headers:
+
+    <san>.idx{b}[.<tag>]       idxN blob, N*K*b/8 bytes
+    <san>.lut_scalar[.<tag>]   float16 [n_groups, 2^b]
+    resA_file / resB_file      float16 [N, rank] / [rank, K]
+
+Nothing here touches the device; the modules are built on the CPU and moved by
+the caller.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import re
+from typing import Dict, Optional, Tuple
+
+import numpy as np
+import torch
+from torch import nn
+
+from palettized_modules import PalettizedLinear, SplitQKV
+
+__all__ = ["validate_indices_layout", "load_palettized_weight", "LAYOUT_AUDIT", "GS_MISMATCHES"]
+
+LAYOUT_AUDIT = {"idx4": 0, "idxN": 0}     # how many members of each kind were validated
+GS_MISMATCHES = []                         # (ctx, recorded gs, derived gs): stale metadata seen
+
+_NAME = re.compile(r"^(?P<base>.*)\.idx(?P<bits>[1-4])(?P<tag>\.[^.]+)?$")
+
+
+def _bits_of_layout(layout) -> int:
+    if isinstance(layout, str) and layout.startswith("idx") and layout[3:].isdigit() \
+            and int(layout[3:]) in (1, 2, 3, 4):
+        return int(layout[3:])
+    raise ValueError(f"not an idxN layout name: {layout!r}")
+
+
+def _is_idxn_artifact_name(name) -> bool:
+    return isinstance(name, str) and "/" not in name and _NAME.match(name) is not None
+
+
+def _bits_of_artifact_name(name) -> int:
+    m = _NAME.match(str(name))
+    if m is None:
+        raise ValueError(f"not an idxN artifact name: {name!r}")
+    return int(m.group("bits"))
+
+
+def _lut_name_of(name) -> Optional[str]:
+    """'<san>.idx{b}' -> '<san>.lut_scalar', '<san>.idx{b}.<tag>' -> '<san>.lut_scalar.<tag>'."""
+    m = _NAME.match(str(name)) if name else None
+    return None if m is None else m.group("base") + ".lut_scalar" + (m.group("tag") or "")
+
+
+def validate_indices_layout(meta: Dict, ctx: str) -> None:
+    """The layout string, the file name and the bitwidth field must agree on one
+    idxN width; anything else is refused, because a blob read at the wrong width
+    has the right byte count and decodes to garbage."""
+    raw = meta.get("indices_layout") or meta.get("layout")
+    try:
+        layout_bits = _bits_of_layout(raw)
+    except ValueError:
+        raise ValueError(f"{ctx}: indices_layout={raw!r} is not an idxN layout ('idx1'..'idx4'); "
+                         f"older artifact formats are not readable, re-run palettization")
+    index_file = str(meta.get("index_file", ""))
+    if not _is_idxn_artifact_name(index_file):
+        raise ValueError(f"{ctx}: index file {index_file!r} is not an idxN artifact")
+    if _bits_of_artifact_name(index_file) != layout_bits:
+        raise ValueError(f"{ctx}: index file {index_file!r} declares "
+                         f"idx{_bits_of_artifact_name(index_file)} but indices_layout={raw!r}")
+    if meta.get("bitwidth") is not None and int(meta["bitwidth"]) != layout_bits:
+        raise ValueError(f"{ctx}: metadata bitwidth {meta['bitwidth']} != the layout's "
+                         f"{layout_bits} bits ({index_file!r})")
+    LAYOUT_AUDIT["idx4" if layout_bits == 4 else "idxN"] += 1
+
+
+def _check_sha(path: str, expected: Optional[str], ctx: str, verify: bool = True) -> None:
+    if not verify or not expected:
+        return
+    h = hashlib.sha256()
+    with open(path, "rb") as f:
+        for chunk in iter(lambda: f.read(1 << 22), b""):
+            h.update(chunk)
+    if h.hexdigest() != expected:
+        raise ValueError(f"{ctx}: SHA256 mismatch for {path} (metadata {expected[:16]}..., "
+                         f"got {h.hexdigest()[:16]}...)")
+
+
+def _read_indices_and_lut(meta: Dict, artifacts_dir: str, ctx: str, shape=None,
+                          verify_sha: bool = True
+                          ) -> Tuple[torch.Tensor, torch.Tensor, int, int, int, int]:
+    """(indices blob, lut [n_groups, 2^b] fp16, bitwidth, group_size, N, K).  The recorded
+    group_size is honoured when n_groups == ceil(N / group_size); otherwise the value
+    derived from the LUT row count is used and the mismatch is noted."""
+    idx_path = os.path.join(artifacts_dir, meta["index_file"])
+    lut_path = os.path.join(artifacts_dir, meta["lut_file"])
+    validate_indices_layout(meta, ctx)
+    _check_sha(idx_path, meta.get("sha256_idx"), ctx, verify_sha)
+    _check_sha(lut_path, meta.get("sha256_lut"), ctx, verify_sha)
+    blob = np.fromfile(idx_path, dtype=np.uint8)
+    lut_np = np.fromfile(lut_path, dtype=np.float16)
+    bits = int(meta["bitwidth"])
+    palette = 1 << bits
+    if lut_np.size % palette:
+        raise ValueError(f"{ctx}: LUT size {lut_np.size} not divisible by palette size {palette}")
+    n_groups = lut_np.size // palette
+    lut = torch.from_numpy(lut_np.copy()).view(n_groups, palette)
+    N, K = shape if shape is not None else meta.get("dense_shape", [None, None])
+    if N is None:
+        raise ValueError(f"{ctx}: metadata missing dense_shape")
+    N, K = int(N), int(K)
+    meta_gs = int(meta["group_size"])
+    if n_groups > 0:
+        derived = (N + n_groups - 1) // n_groups
+        if meta_gs > 0 and n_groups == (N + meta_gs - 1) // meta_gs:
+            group_size = meta_gs
+        else:
+            group_size = derived
+            if meta_gs > 0 and meta_gs != derived:
+                GS_MISMATCHES.append((ctx, meta_gs, derived))
+    else:
+        group_size = meta_gs
+    want = N * ((K * bits + 7) // 8)
+    if blob.size != want:
+        raise ValueError(f"{ctx}: index file {meta['index_file']} has {blob.size} B, expected "
+                         f"N*K*b/8 = {want} B (N={N}, K={K}, bitwidth={bits})")
+    return torch.from_numpy(blob.copy()), lut, bits, group_size, N, K
+
+
+def _read_residual(meta: Dict, artifacts_dir: str, ctx: str, N: int, K: int):
+    res = meta.get("residual")
+    if not res:
+        return None, None
+    a_path = os.path.join(artifacts_dir, res["resA_file"])
+    b_path = os.path.join(artifacts_dir, res["resB_file"])
+    _check_sha(a_path, res.get("sha256_resA"), ctx)
+    _check_sha(b_path, res.get("sha256_resB"), ctx)
+    rank = int(res["rank"])
+    A = torch.from_numpy(np.fromfile(a_path, dtype=np.float16).copy()).view(N, rank)
+    B = torch.from_numpy(np.fromfile(b_path, dtype=np.float16).copy()).view(rank, K)
+    return A, B
+
+
+def _read_stream2(meta: Dict, artifacts_dir: str, ctx: str, N: int, K: int, bitwidth: int,
+                  group_size: int, verify_sha: bool = True):
+    """The second member of a declared "streams" list -> (indices2, lut2, bitwidth2).
+    A declared but missing member is an error, never a silent single-stream load."""
+    streams = meta.get("streams")
+    if not isinstance(streams, list) or len(streams) < 2:
+        raise ValueError(f"{ctx}: metadata 'streams' must be a list with at least 2 entries, "
+                         f"got {streams!r}")
+    base = streams[0] if isinstance(streams[0], dict) else {}
+    if base.get("file") != meta.get("index_file"):
+        raise ValueError(f"{ctx}: streams[0] file {base.get('file')!r} != the meta's index_file "
+                         f"{meta.get('index_file')!r}; the first entry must describe the base "
+                         f"stream")
+    entry = streams[1]
+    if not isinstance(entry, dict) or "file" not in entry:
+        raise ValueError(f"{ctx}: stream-2 entry must be a dict carrying 'file' (got {entry!r})")
+    idx2 = str(entry["file"])
+    if not _is_idxn_artifact_name(idx2):
+        raise ValueError(f"{ctx}: stream-2 file {idx2!r} is not a (tagged) idxN artifact name")
+    if entry.get("bitwidth") is not None:
+        bits2 = int(entry["bitwidth"])
+        if bits2 != _bits_of_artifact_name(idx2):
+            raise ValueError(f"{ctx}: stream-2 entry bitwidth {bits2} != the file name's "
+                             f"idx{_bits_of_artifact_name(idx2)} ({idx2!r})")
+    else:
+        bits2 = _bits_of_artifact_name(idx2)
+    lut2 = _lut_name_of(idx2)
+    for fname in (idx2, lut2):
+        if not os.path.exists(os.path.join(artifacts_dir, fname)):
+            raise ValueError(f"{ctx}: metadata declares {len(streams)} streams but stream-2 "
+                             f"member {fname!r} is missing from {artifacts_dir}; the two-stream "
+                             f"artifact set is incomplete")
+    member = {"index_file": idx2, "lut_file": lut2, "sha256_idx": entry.get("sha256"),
+              "sha256_lut": entry.get("sha256_lut"), "bitwidth": bits2,
+              "group_size": int(entry.get("gs", group_size)), "indices_layout": f"idx{bits2}"}
+    indices2, lut2_t, _, _, _, _ = _read_indices_and_lut(member, artifacts_dir, f"{ctx}:stream2",
+                                                         shape=(N, K), verify_sha=verify_sha)
+    if entry.get("n_groups") is not None and int(entry["n_groups"]) != lut2_t.shape[0]:
+        raise ValueError(f"{ctx}: stream-2 n_groups {entry['n_groups']} != the LUT's "
+                         f"{lut2_t.shape[0]} rows")
+    return indices2, lut2_t, bits2
+
+
+def _awq_for(meta: Dict, awq_scales: Optional[Dict]):
+    """(scale tensor or None, fold order or None) for one tensor record."""
+    rec = meta.get("awq") or {}
+    s = None
+    if awq_scales:
+        s = awq_scales.get(meta.get("var")) or awq_scales.get(meta.get("name"))
+    return s, rec.get("fold_order")
+
+
+def _build(meta, artifacts_dir, ctx, shape, residual, reference, verify_sha, awq_s, fold, bias):
+    indices, lut, bw, gs, N, K = _read_indices_and_lut(meta, artifacts_dir, ctx, shape, verify_sha)
+    resA = resB = None
+    if residual:
+        resA, resB = _read_residual(meta, artifacts_dir, ctx, N, K)
+    indices2 = lut2 = bw2 = None
+    if meta.get("streams"):
+        indices2, lut2, bw2 = _read_stream2(meta, artifacts_dir, ctx, N, K, bw, gs, verify_sha)
+    rot = meta.get("rotation")
+    return PalettizedLinear(indices, lut, bw, gs, N, K, bias=bias, resA=resA, resB=resB,
+                            indices2=indices2, lut2=lut2, bitwidth2=bw2, reference=reference,
+                            rotation_seed=rot["seed"] if rot else None,
+                            rotation_k=rot["k"] if rot else None, awq_scale=awq_s,
+                            fold_order=fold)
+
+
+def load_palettized_weight(tensor_meta: Dict, artifacts_dir: str, bias=None,
+                           residual: bool = False, reference: bool = False,
+                           verify_sha: bool = True, awq_scales: Optional[Dict] = None):
+    """PalettizedLinear for a plain record, SplitQKV for a record with "components"
+    (Q, K, V members share K; each N comes from its packed_len_bytes; a bias is sliced
+    per component)."""
+    var = tensor_meta.get("var", "?")
+    awq_s, fold = _awq_for(tensor_meta, awq_scales)
+    if "components" not in tensor_meta:
+        return _build(tensor_meta, artifacts_dir, var, None, residual, reference, verify_sha,
+                      awq_s, fold, None if bias is None else bias.clone())
+    K = int(tensor_meta["dense_shape"][1])
+    comps = []
+    for name in ("Q", "K", "V"):
+        cm = tensor_meta["components"][name]
+        n = int(cm["packed_len_bytes"]) * 8 // (K * int(cm["bitwidth"]))
+        comps.append(_build(cm, artifacts_dir, f"{var}:{name}", (n, K), residual, reference,
+                            verify_sha, awq_s, fold, None))
+    if bias is not None:
+        off = 0
+        for m in comps:
+            m.bias = nn.Parameter(bias[off:off + m.N].clone())
+            off += m.N
+        if off != bias.shape[0]:
+            raise ValueError(f"{var}: bias length {bias.shape[0]} != sum of component N ({off})")
+    return SplitQKV(*comps)

@@ -477,6 +477,102 @@ class FusedPalettizedMLP(nn.Module):
         return state
 
 
+class SplitQKV(nn.Module):
+    """Three palettized projections that share their input, concatenated along the
+    output axis (upstream :1390-1641).  One token takes one grouped launch that
+    writes the three outputs side by side into a persistent [1, Nq+Nk+Nv] row; every
+    other shape is the per-module chain plus torch.cat."""
+
+    def __init__(self, q_proj, k_proj, v_proj):
+        super().__init__()
+        self.q_proj, self.k_proj, self.v_proj = q_proj, k_proj, v_proj
+        self._merge_state = None
+
+    def forward(self, x):
+        y = self._gemv_multi_decode(x)
+        if y is not None:
+            return y
+        return torch.cat([self.q_proj(x), self.k_proj(x), self.v_proj(x)], dim=-1)
+
+    def _gemv_multi_decode(self, x):
+        if _env_on("FLUTE_NO_MERGE"):
+            return None
+        lead = None
+        if x.dim() == 3:
+            if x.shape[0] * x.shape[1] != 1:
+                return None
+            lead = (x.shape[0], x.shape[1])
+            x = x.reshape(1, x.shape[2])
+        if x.dim() != 2 or x.shape[0] != 1 or not x.is_cuda or not x.is_contiguous() \
+                or x.requires_grad or x.dtype not in (torch.float16, torch.bfloat16):
+            return None
+        state = self._merge_state
+        if state is None or state["device"] != x.device or state["dtype"] != x.dtype:
+            state = self._merge_state = self._build_state(x.device, x.dtype)
+        if not state["ok"]:
+            return None
+        _count("gemv_multi")
+        _flute().qgemm_gemv_multi(x, state["seg_table"], lut_dtype=self.q_proj.lut.dtype)
+        y = state["out"]
+        return y.view(lead[0], lead[1], y.shape[1]) if lead is not None else y
+
+    def _build_state(self, device, dtype):
+        members = (self.q_proj, self.k_proj, self.v_proj)
+        state = {"ok": False, "device": device, "dtype": dtype}
+
+        def refuse(why):
+            state["reason"] = why
+            return state
+
+        if not all(isinstance(m, PalettizedLinear) for m in members):
+            return refuse("non-PalettizedLinear member")
+        if any(m.reference for m in members):
+            return refuse("reference member")
+        if len({m.K for m in members}) != 1 or any(m.N % 128 for m in members):
+            return refuse("K mismatch or ragged N")
+        if len({m.lut.dtype for m in members}) != 1 or \
+                members[0].lut.dtype not in (torch.float16, torch.bfloat16):
+            return refuse("lut dtype")
+        rot = [m.rot_signs is not None for m in members]
+        if any(rot) and not all(rot):
+            return refuse("mixed rotation presence")
+        fx = _flute()
+        total = sum(m.N for m in members)
+        out = torch.zeros(1, total, dtype=dtype, device=device)
+        rows, keep, specs, off = [], [], [], 0
+        esize = out.element_size()
+        for m in members:
+            fused = m._fusable(torch.empty(0, dtype=dtype), fx.GEMV_SPLITK_MAX_RESIDUAL_RANK)
+            if fused is None:
+                return refuse("residual/bias contract")
+            resB, resA, bias = fused
+            signs = awq = None
+            if m.rot_signs is not None:
+                if m._rotation_backend() != "auto":
+                    return refuse("pinned rotation backend")
+                signs = m._signs_on(device).contiguous()
+                awq = m._awq_scale_on(device) if m._compensated() else None
+            b2 = m.bitwidth2 if m.has_stream2 else 0
+            ptr = lambda t: 0 if t is None else t.data_ptr()
+            rank = 0 if resB is None else int(resB.shape[0])
+            rows.append([ptr(m.indices), ptr(m.lut), ptr(m.indices2) if b2 else 0,
+                         ptr(m.lut2) if b2 else 0, ptr(resB), ptr(resA), ptr(bias),
+                         out.data_ptr() + off * esize, m.N, rank, m.bitwidth, b2, m.group_size,
+                         ptr(signs), ptr(awq)])
+            keep.append((signs, awq))
+            specs.append((m.bitwidth, b2, m.group_size, m.N, rank))
+            off += m.N
+        if (out.data_ptr() % 16) or any((r[7] % 16) for r in rows):
+            return refuse("output slices are not 16-byte aligned")
+        if not fx.gemv_multi_supported(members[0].K, total // 128,
+                                       [(b1, b2, gs) for b1, b2, gs, _, _ in specs],
+                                       sum(r for _, _, _, _, r in specs), all(rot)):
+            return refuse("extension/gate: multi")
+        state.update(ok=True, seg_table=torch.tensor(rows, dtype=torch.int64), out=out,
+                     keepalive=keep, specs=specs)
+        return state
+
+
 def act_name(fn) -> str:
     name = getattr(fn, "__name__", None) or type(fn).__name__
     return name.lower().replace("activation", "")

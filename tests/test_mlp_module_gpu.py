@@ -197,3 +197,26 @@ def test_gemm_with_rotation_through_the_c_abi():
         # LUT's fp16 (exact for these magnitudes)
         ref = _exact(w, xr.to(torch.bfloat16).half()).to(torch.bfloat16)
         assert rel_l2(C.cpu(), ref) <= 4e-3
+
+
+@pytest.mark.parametrize("rot", [False, True])
+def test_split_qkv_module(rot):
+    """One token: one grouped launch writes Q|K|V side by side; several tokens: the
+    per-module chain and a concatenation.  Both against the reference-mode modules."""
+    K = 1024
+    ws = [make_weight(512, K, seed=1), make_weight(256, K, bits=3, gs=64, bits2=3, rank=8, seed=2),
+          make_weight(256, K, bits=4, gs=128, bias=True, seed=3)]
+    kw = dict(rotation_seed=4, rotation_k=K) if rot else {}
+    pairs = [_modules(w, **kw) for w in ws]
+    ref = pm.SplitQKV(*[p[0] for p in pairs])
+    ker = pm.SplitQKV(*[p[1] for p in pairs])
+    x = make_x(1, K, seed=5)
+    pm.ROUTE_CENSUS.clear()
+    y = ker(x.to(DEV).reshape(1, 1, K))
+    assert y.shape == (1, 1, 1024)
+    assert pm.ROUTE_CENSUS.get("gemv_multi") == 1 and ker._merge_state["ok"], ker._merge_state
+    assert rel_l2(y.cpu().reshape(1, -1), ref(x)) <= TOL
+    y2 = ker(x.to(DEV))                                  # persistent output, same values
+    assert torch.equal(y2.cpu(), y.cpu().reshape(1, -1))
+    xs = make_x(5, K, seed=6)
+    assert rel_l2(ker(xs.to(DEV)).cpu(), ref(xs)) <= 2e-3
