@@ -104,6 +104,64 @@ def _cpu_baseline(torch, seconds_budget=20.0):
                       f"os.cpu_count={os.cpu_count()}"}
 
 
+def _gemv_section(torch, _lib, ctypes, sets, gen, dev, O):
+    """The other M = 1 configurations beside the headline block, each parity-gated against
+    the oracle on the rows of one tile: the north-star GEMV 4096 -> 12288 (GB/s on packed
+    index + LUT bytes, the numerator the target is stated on), the same GEMV with the
+    block-128 Hadamard rotation fused into its prologue, and the narrow split-K shapes."""
+    out = {}
+    act = torch.bfloat16
+    x = torch.randn(1, H, device=dev, generator=gen).to(act)
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+
+    def run(name, descs, N, K, xin, keep, signs=None, block=0):
+        y = torch.zeros(1, N, dtype=act, device=dev)
+
+        def call(i):
+            st = _lib.lib.flute_gemv(ctypes.byref(descs[i % len(descs)]), xin.data_ptr(),
+                                     y.data_ptr(), _lib.BF16, 0, stream())
+            if st != 0:
+                raise RuntimeError(_lib.last_error())
+
+        call(0)
+        torch.cuda.synchronize()
+        blob, lut = keep[0]
+        per = (K // 64) * 4096
+        tile = (N // 128) // 2
+        Wt = O.dequant(blob[tile * per:(tile + 1) * per].cpu().numpy(), lut[tile:tile + 1].cpu(),
+                       128, K, GS, 4).double()
+        xr = xin.cpu()
+        if signs is not None:
+            xr = O.block_fht_reference(xr, block, signs.cpu()).to(act)
+        ref = xr.double() @ Wt.t()
+        got = y[:, tile * 128:(tile + 1) * 128].cpu().double()
+        err = float(((got - ref) ** 2).sum() / (ref ** 2).sum()) ** 0.5
+        if err > 4e-3:
+            raise SystemExit(f"bench.py: parity gate failed for {name} ({err:.2e})")
+        n = 96
+        us = _time_graph(torch, lambda: [call(i) for i in range(n)]) / n * 1e3
+        wbytes = N * K // 2 + (N // GS) * 32
+        out[name] = {"us_per_call": round(us, 2), "gbs_index_plus_lut": round(wbytes / us / 1e3, 1),
+                     "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                     "parity_rel_l2": err}
+
+    gate = [s["g"] for s in sets]
+    keep = [s["t"][0] for s in sets]
+    run("gemv_4096x12288", gate, I, H, x, keep)
+    signs = (torch.randint(0, 2, (H,), device=dev, generator=gen).float() * 2 - 1).contiguous()
+    rot = []
+    for s in sets:
+        d = _lib.FluteLinear()
+        ctypes.memmove(ctypes.byref(d), ctypes.byref(s["g"]), ctypes.sizeof(d))
+        d.signs, d.rot_block = signs.data_ptr(), 128
+        rot.append(d)
+    run("gemv_4096x12288_fht128_fused", rot, I, H, x, keep, signs=signs, block=128)
+    for N in (1024, 512):
+        ws = [_weights(torch, N, H, gen, dev, torch.float16) for _ in range(16)]
+        run(f"gemv_split_k_4096x{N}", [_desc(_lib, b, l, N, H) for b, l in ws], N, H, x, ws)
+    return out
+
+
 def _gemm_section(torch, _lib, ctypes, sets, gen, dev, O):
     """The second half of the metric: C[M, 12288] = A[M, 4096] @ W^T on the same idx4
     blobs (the gate projections of the weight sets), bf16 LUT, bf16 activations, bf16
@@ -164,6 +222,7 @@ def main():
     ap.add_argument("--sets", type=int, default=12, help="distinct weight sets (72 MiB each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M>1 LUT-GEMM section")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other M=1 configurations")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 64 MiB device copy, so that a counter run of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE/WRITE_SIZE by")
@@ -270,6 +329,7 @@ def main():
     achieved = bytes_gate_up / (ms_gu * 1e-3) / 1e9
 
     gemm = None if args.no_gemm else _gemm_section(torch, _lib, ctypes, sets, gen, dev, O)
+    extra = None if args.no_extra else _gemv_section(torch, _lib, ctypes, sets, gen, dev, O)
 
     out = {
         "metric": "M=1 LUT-GEMV achieved HBM GB/s (% of peak); M=256 LUT-GEMM TFLOP/s (% MFMA)",
@@ -291,6 +351,8 @@ def main():
     }
     if gemm is not None:
         out["gemm"] = gemm
+    if extra is not None:
+        out["other_m1_configs"] = extra
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = _cpu_baseline(torch)
     print(json.dumps(out))

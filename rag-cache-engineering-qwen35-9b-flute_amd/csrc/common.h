@@ -79,11 +79,8 @@ __device__ __forceinline__ uint16_t f2h(float f) {     // round to nearest even
 __device__ __forceinline__ float bf2f(uint16_t h) {
     return __builtin_bit_cast(float, (uint32_t)h << 16);
 }
-__device__ __forceinline__ uint16_t f2bf(float f) {    // round to nearest even, NaN kept quiet
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+__device__ __forceinline__ uint16_t f2bf(float f) {    // round to nearest even (v_cvt_pk_bf16_f32)
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float load_act(const void *p, int64_t i, int is_bf16) {
     uint16_t h = ((const uint16_t *)p)[i];

@@ -51,23 +51,47 @@ __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
             count = 1 << nstages;
         }
         const float inv = inv_sqrt_pow2(nstages);
-        for (int j = tid; j < count; j += kFhtThreads) {
-            float f = load_any(p.x, row + off + j, p.dtype);
-            if (p.adjoint) f *= p.signs[off + j];
-            else if (p.awq) f *= p.awq[off + j];
-            buf[fht_slot(j)] = f;
+        // Eight columns per thread and step; the loads of a step (row, signs, scale) are
+        // independent and issued together, so each phase is one memory round trip.
+#pragma unroll 2
+        for (int j = tid * 8; j < count; j += kFhtThreads * 8) {
+            float f[8], m[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) f[q] = load_any(p.x, row + off + j + q, p.dtype);
+            if (p.adjoint || p.awq) {
+                const float *mul = p.adjoint ? p.signs : p.awq;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) m[q] = mul[off + j + q];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) f[q] *= m[q];
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) buf[fht_slot(j + q)] = f[q];
         }
         __syncthreads();
         fht_lds(buf, count, nstages, tid, kFhtThreads);
-        for (int j = tid; j < count; j += kFhtThreads) {
-            float t = buf[fht_slot(j)];
-            if (p.adjoint) {
-                t = t * inv;
-            } else {
-                t = t * p.signs[off + j] * inv;
-                if (p.awq) t = t / p.awq[off + j];
+#pragma unroll 2
+        for (int j = tid * 8; j < count; j += kFhtThreads * 8) {
+            float sg[8], sc[8];
+            if (!p.adjoint) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) sg[q] = p.signs[off + j + q];
+                if (p.awq) {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) sc[q] = p.awq[off + j + q];
+                }
             }
-            store_any(p.out, row + off + j, p.dtype, t);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                float t = buf[fht_slot(j + q)];
+                if (p.adjoint) {
+                    t = t * inv;
+                } else {
+                    t = t * sg[q] * inv;
+                    if (p.awq) t = t / sc[q];
+                }
+                store_any(p.out, row + off + j + q, p.dtype, t);
+            }
         }
         __syncthreads();
         off += count;

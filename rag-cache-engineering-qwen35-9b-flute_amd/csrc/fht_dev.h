@@ -63,16 +63,20 @@ __device__ __forceinline__ void fht_pass(float *buf, int b, int sh0, int tid, in
 // count / b independent blocks of b = 2^nstages consecutive values (count a
 // multiple of b; b >= 2).  Must be called by every thread of the workgroup; the
 // buffer must be complete (barrier) on entry and is complete on exit.
+template <int RMAX = 4>
 __device__ __forceinline__ void fht_lds(float *buf, int count, int nstages, int tid,
                                         int nthreads) {
+    // RMAX = stages per pass: 4 keeps 16 values in registers, 3 keeps 8 (for callers
+    // that are short of registers); the order of the stages, and so every bit of the
+    // result, is the same.
     int sh0 = 0;
-    while (nstages - sh0 >= 4) {
-        fht_pass<4>(buf, count, sh0, tid, nthreads);
+    while (nstages - sh0 >= RMAX) {
+        fht_pass<RMAX>(buf, count, sh0, tid, nthreads);
         __syncthreads();
-        sh0 += 4;
+        sh0 += RMAX;
     }
     const int rem = nstages - sh0;
-    if (rem == 3) fht_pass<3>(buf, count, sh0, tid, nthreads);
+    if (RMAX > 3 && rem == 3) fht_pass<3>(buf, count, sh0, tid, nthreads);
     else if (rem == 2) fht_pass<2>(buf, count, sh0, tid, nthreads);
     else if (rem == 1) fht_pass<1>(buf, count, sh0, tid, nthreads);
     if (rem) __syncthreads();

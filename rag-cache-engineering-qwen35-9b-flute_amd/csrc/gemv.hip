@@ -36,6 +36,7 @@ struct Plan {
         const uint16_t *resB;
         const float *signs, *awq;
         int R, seg;
+        int share;              // index of an earlier entry with the same rotation, or -1
         size_t xb_off, xrot_off;
     } pre[kGemvMaxSegs];
     int npre;
@@ -178,7 +179,13 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
             col += (w.N / 128) * spt;
             ticket += (w.N / 128) * spt;
         }
-        if (w.R > 0) {
+        // Rotating inside the GEMV makes every workgroup transform the whole row itself
+        // (about 5 us of VALU work per CU at K = 4096); a separate rotation launch in
+        // front measured slower still (a dependent launch costs more than that), so it
+        // stays an opt-in.
+        const bool prerotate = w.signs != nullptr && w.R == 0 &&
+                               env_int("FLUTE_GEMV_PREROTATE", 0) != 0;
+        if (w.R > 0 || prerotate) {
             // the residual needs x . resB[r] before any row can finish: computed by a
             // small kernel in front, on the rotated input when the weight is rotated
             Plan::Pre &pre = plan->pre[plan->npre++];
@@ -188,9 +195,12 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
             pre.R = w.R;
             pre.seg = i;
             pre.xb_off = xb_off;
-            pre.xrot_off = xrot_off;
+            pre.share = -1;
+            for (int j = 0; j + 1 < plan->npre && w.signs; ++j)
+                if (plan->pre[j].signs == w.signs && plan->pre[j].awq == w.awq) pre.share = j;
+            pre.xrot_off = pre.share >= 0 ? plan->pre[pre.share].xrot_off : xrot_off;
             xb_off += (size_t)((w.R + 3) & ~3);
-            if (w.signs) xrot_off += (size_t)K;
+            if (w.signs && pre.share < 0) xrot_off += (size_t)K;
             sg.signs = nullptr;                     // the kernel reads the pre-rotated row
             sg.awq = nullptr;
         } else {
@@ -366,17 +376,21 @@ flute_status launch(Plan &plan, int act_dtype, hipStream_t stream) {
             const uint16_t *xin = plan.p.x;
             if (pre.signs) {
                 uint16_t *xr = xrot_base + pre.xrot_off;
-                st = flute_fht(plan.p.x, pre.signs, pre.awq, xr, 1, plan.p.K, act_dtype, 0,
-                               plan.rot_block, stream);
-                if (st != FLUTE_OK) return st;
+                if (pre.share < 0) {
+                    st = flute_fht(plan.p.x, pre.signs, pre.awq, xr, 1, plan.p.K, act_dtype, 0,
+                                   plan.rot_block, stream);
+                    if (st != FLUTE_OK) return st;
+                }
                 xin = xr;
                 plan.p.seg[pre.seg].xsrc = xr;
             }
-            float *xb = xb_base + pre.xb_off;
-            hipLaunchKernelGGL(residual_coeff_kernel, dim3(pre.R), dim3(256), 0, stream, xin,
-                               pre.resB, xb, plan.p.K, plan.p.act_bf16);
-            FLUTE_HIP_CHECK(hipGetLastError());
-            plan.p.seg[pre.seg].xb = xb;
+            if (pre.R > 0) {
+                float *xb = xb_base + pre.xb_off;
+                hipLaunchKernelGGL(residual_coeff_kernel, dim3(pre.R), dim3(256), 0, stream, xin,
+                                   pre.resB, xb, plan.p.K, plan.p.act_bf16);
+                FLUTE_HIP_CHECK(hipGetLastError());
+                plan.p.seg[pre.seg].xb = xb;
+            }
         }
     }
     return plan.lut_bf16 ? launch_width<true>(plan, stream) : launch_width<false>(plan, stream);

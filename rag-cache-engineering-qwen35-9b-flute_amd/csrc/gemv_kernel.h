@@ -260,6 +260,53 @@ __device__ __forceinline__ uint4 to_compute_type(uint4 v, int act_bf16) {
     return v;
 }
 
+// Output side of the fused rotation, eight columns per step: value * sign * inv
+// (/ awq), rounded to the activation type exactly as the standalone kernel rounds,
+// then converted to the compute type.  The eight sign (and scale) loads of a step are
+// independent and issued together, so a step costs one memory round trip, not eight.
+template <bool BF16>
+__device__ __forceinline__ void rotated_out8(const float *buf, int j, const float *signs,
+                                             const float *awq, int g, float inv, int act_bf16,
+                                             uint16_t *dst) {
+    float sg[8], sc[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) sg[q] = signs[g + q];
+    if (awq) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sc[q] = awq[g + q];
+    }
+    uint32_t o[4];
+    const int s0 = fht_slot(j);                        // j is a multiple of 8: slot(j + q) = s0 ^ q
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        float t = buf[s0 ^ q] * sg[q] * inv;
+        if (awq) t = t / sc[q];
+        const uint16_t a = round_act(t, act_bf16);
+        const float back = act_bf16 ? bf2f(a) : h2f(a);
+        const uint32_t h = BF16 ? f2bf(back) : f2h(back);
+        if (q & 1) o[q >> 1] |= h << 16;
+        else o[q >> 1] = h;
+    }
+    *(uint4 *)dst = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// Input side: eight activations (times the scale when compensated) into the swizzled
+// fp32 buffer.
+__device__ __forceinline__ void rotated_in8(float *buf, int j, const uint16_t *x, int g,
+                                            const float *awq, int act_bf16) {
+    float f[8], sc[8];
+    load_act8(x, g, act_bf16, f);
+    if (awq) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sc[q] = awq[g + q];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) f[q] *= sc[q];
+    }
+    const int s0 = fht_slot(j);                        // j is a multiple of 8: slot(j + q) = s0 ^ q
+#pragma unroll
+    for (int q = 0; q < 8; ++q) buf[s0 ^ q] = f[q];
+}
+
 // Stage the activation slice [k0, k0 + kc) into LDS as 16-bit values of the
 // compute type (the LUT's type), 16 bytes per thread per step so that the whole
 // slice is one round trip to memory.  With signs, the rotation of every segment
@@ -280,26 +327,16 @@ __device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *sig
     float *buf = (float *)lds;
     if (p.fht_block > 0) {
         // equal blocks: the slice is a whole number of blocks
-        for (int j = tid * 8; j < kc; j += nthreads * 8) {
-            float f[8];
-            load_act8(x, k0 + j, p.act_bf16, f);
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                if (awq) f[q] *= awq[k0 + j + q];
-                buf[fht_slot(j + q)] = f[q];
-            }
-        }
+#pragma unroll 2
+        for (int j = tid * 8; j < kc; j += nthreads * 8)
+            rotated_in8(buf, j, x, k0 + j, awq, p.act_bf16);
         __syncthreads();
         const int nst = 31 - __builtin_clz((unsigned)p.fht_block);
         fht_lds(buf, kc, nst, tid, nthreads);
         const float inv = inv_sqrt_pow2(nst);
-        for (int j = tid; j < kc; j += nthreads) {
-            float t = buf[fht_slot(j)] * signs[k0 + j] * inv;
-            if (awq) t = t / awq[k0 + j];
-            const uint16_t a = round_act(t, p.act_bf16);
-            const float back = p.act_bf16 ? bf2f(a) : h2f(a);
-            xs[j] = BF16 ? f2bf(back) : f2h(back);
-        }
+#pragma unroll 2
+        for (int j = tid * 8; j < kc; j += nthreads * 8)
+            rotated_out8<BF16>(buf, j, signs, awq, k0 + j, inv, p.act_bf16, xs + j);
         __syncthreads();
         return;
     }
@@ -309,25 +346,16 @@ __device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *sig
         const int b = 1 << nst;
         const int lo = max(off, k0), hi = min(off + b, k0 + kc);
         if (lo < hi) {                             // uniform across the workgroup
-            for (int j = tid * 8; j < b; j += nthreads * 8) {
-                float f[8];
-                load_act8(x, off + j, p.act_bf16, f);
-#pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    if (awq) f[q] *= awq[off + j + q];
-                    buf[fht_slot(j + q)] = f[q];
-                }
-            }
+#pragma unroll 2
+            for (int j = tid * 8; j < b; j += nthreads * 8)
+                rotated_in8(buf, j, x, off + j, awq, p.act_bf16);
             __syncthreads();
             fht_lds(buf, b, nst, tid, nthreads);
             const float inv = inv_sqrt_pow2(nst);
-            for (int k = lo + tid; k < hi; k += nthreads) {
-                float t = buf[fht_slot(k - off)] * signs[k] * inv;
-                if (awq) t = t / awq[k];
-                const uint16_t a = round_act(t, p.act_bf16);
-                const float back = p.act_bf16 ? bf2f(a) : h2f(a);
-                xs[k - k0] = BF16 ? f2bf(back) : f2h(back);
-            }
+            // lo, hi, off are multiples of 8 (segments and slices are multiples of 32)
+#pragma unroll 2
+            for (int k = lo + tid * 8; k < hi; k += nthreads * 8)
+                rotated_out8<BF16>(buf, k - off, signs, awq, k, inv, p.act_bf16, xs + (k - k0));
             __syncthreads();                       // scratch is reused by the next segment
         }
         off += b;
