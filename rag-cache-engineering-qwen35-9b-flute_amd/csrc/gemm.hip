@@ -67,7 +67,12 @@ flute_status launch_gemm_bits(const GemmParams &p, dim3 grid, int lds, hipStream
             default: return launch_gemm<MB, KW, MW, BF16, 1>(p, grid, lds, stream);
         }
     }
-    return launch_gemm<MB, KW, MW, BF16, 0>(p, grid, lds, stream);
+    if constexpr (MB == 1) {
+        return launch_gemm<MB, KW, MW, BF16, 0>(p, grid, lds, stream);
+    } else {
+        set_error("flute_gemm: two streams at this size run as one launch per stream");
+        return FLUTE_ERR_UNSUPPORTED;
+    }
 }
 
 template <bool BF16>
@@ -79,6 +84,39 @@ flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 gri
 }
 
 #endif
+
+// LDS plan of one launch: pair tables (+ staging on the fast path), sized against the
+// reduction tree and the totals tile that reuse the same memory afterwards.
+// A single 4-bit stream with at most two LUT groups per 128-row tile gets 64-lane
+// replication (256 bytes per entry, 64 KB per group, first table at LDS offset 0: the
+// layout the one-instruction address needs).  Everything else: as much replication as
+// the budget allows, 32 lanes at most.
+int plan_lds(GemmParams &p, const GemmShape &shape) {
+    const int ngrp = p.gs >= 128 ? 1 : 128 / p.gs;
+    const bool perm = p.nstreams == 1 && p.bits[0] == 4 && ngrp <= 2 &&
+                      getenv("FLUTE_GEMM_NO_PERM") == nullptr;
+    const int table_budget = (shape.mb == 1 ? 64 : 96) * 1024 / p.nstreams;
+    int lds_tables = 0;
+    for (int s = 0; s < p.nstreams; ++s) {
+        const int entries = ngrp << (2 * p.bits[s]);
+        int rl = 5;
+        while (rl > 0 && (entries << rl) * 4 > table_budget) --rl;
+        if (perm) rl = 6;
+        p.rep_log2[s] = rl;
+        p.tab_off[s] = lds_tables;
+        lds_tables += (entries << rl) * 4;
+    }
+    if (perm) {                                  // per-wavefront tile staging behind the tables
+        p.stage_off = lds_tables;
+        lds_tables += shape.kw * shape.mw * 4096;
+    }
+    const int slot_bytes = shape.mb * 8 * 64 * 16;
+    const int lds_reduce = (shape.kw / 2) * shape.mw * slot_bytes;
+    const int lds_tile = shape.mw * shape.mb * 16 * 132 * 4 + 16;   // totals tile + ticket flag
+    int lds = lds_tables > lds_reduce ? lds_tables : lds_reduce;
+    if (lds_tile > lds) lds = lds_tile;
+    return lds;
+}
 
 }  // namespace
 
@@ -131,37 +169,6 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     p.vec_store = (ldc % 8 == 0) && (((uintptr_t)C & 15) == 0);
     p.mblk_total = (M + 15) / 16;
 
-    // ---- pair tables ---------------------------------------------------------------
-    // A single 4-bit stream with at most two LUT groups per 128-row tile gets 64-lane
-    // replication (256 bytes per entry, 64 KB per group, first table at LDS offset 0:
-    // the layout the one-instruction address needs).  Everything else: as much
-    // replication as the budget allows, 32 lanes at most.
-    const int ngrp = w->group_size >= 128 ? 1 : 128 / w->group_size;
-    const bool perm = p.nstreams == 1 && p.bits[0] == 4 && ngrp <= 2 &&
-                      getenv("FLUTE_GEMM_NO_PERM") == nullptr;
-    const int table_budget = (shape.mb == 1 ? 64 : 96) * 1024 / p.nstreams;
-    int lds_tables = 0;
-    for (int s = 0; s < p.nstreams; ++s) {
-        const int entries = ngrp << (2 * p.bits[s]);
-        int rl = 5;
-        while (rl > 0 && (entries << rl) * 4 > table_budget) --rl;
-        if (perm) rl = 6;
-        p.rep_log2[s] = rl;
-        p.tab_off[s] = lds_tables;
-        lds_tables += (entries << rl) * 4;
-    }
-    if (perm) {                                  // per-wavefront tile staging behind the tables
-        p.stage_off = lds_tables;
-        lds_tables += shape.kw * shape.mw * 4096;
-    }
-    const int slot_bytes = shape.mb * 8 * 64 * 16;
-    const int lds_reduce = (shape.kw / 2) * shape.mw * slot_bytes;
-    const int lds_tile = shape.mw * shape.mb * 16 * 132 * 4 + 16;   // totals tile + ticket flag
-    int lds = lds_tables > lds_reduce ? lds_tables : lds_reduce;
-    if (lds_tile > lds) lds = lds_tile;
-    FLUTE_REQUIRE(lds <= kLdsPerCU, FLUTE_ERR_UNSUPPORTED,
-                  "flute_gemm: %d bytes of LDS exceed the %d of one CU", lds, kLdsPerCU);
-
     // ---- grid and K split --------------------------------------------------------
     const int tiles = w->N / 128;
     const int mchunks = (p.mblk_total + shape.mb * shape.mw - 1) / (shape.mb * shape.mw);
@@ -182,7 +189,8 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
 
     // ---- workspace: [partial images][xb][Ap] -----------------------------------------
     const size_t image = (size_t)shape.mw * shape.mb * 8 * 64 * 4;
-    const size_t p_floats = ksplit > 1 ? (size_t)ksplit * units * image : 0;
+    const int zparts = ksplit * ((p.nstreams == 2 && shape.mb > 1) ? 2 : 1);
+    const size_t p_floats = zparts > 1 ? (size_t)zparts * units * image : 0;
     const size_t xb_floats = ((size_t)M * w->R + 3) & ~(size_t)3;
     const size_t ap_floats = (size_t)p.G * 2 * p.mblk_pad * 64 * 4;
     const size_t rot_floats = w->signs ? ((size_t)M * w->K / 2 + 4) & ~(size_t)3 : 0;
@@ -225,7 +233,29 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
 #ifdef FLUTE_GEMM_TRACE
     if (const char *e = getenv("FLUTE_GEMM_TRACE_PTR")) p.trace = (unsigned long long *)strtoull(e, nullptr, 10);
 #endif
+    // Two streams with four blocks per wavefront: one launch per stream through the
+    // single-stream kernels (the two-stream kernel does not fit the register file at
+    // that size); both write partial tiles and the last workgroup of the second launch
+    // folds everything, exactly as a K split does.
+    const bool per_stream = p.nstreams == 2 && shape.mb > 1;
+    const int passes = per_stream ? 2 : 1;
     const dim3 grid(tiles, mchunks, ksplit);
-    if (w->lut_dtype == FLUTE_BF16) return launch_gemm_shape<true>(shape, p, grid, lds, stream);
-    return launch_gemm_shape<false>(shape, p, grid, lds, stream);
+    for (int pass = 0; pass < passes; ++pass) {
+        GemmParams q = p;
+        if (per_stream) {
+            q.nstreams = 1;
+            q.q[0] = p.q[pass];
+            q.lut[0] = p.lut[pass];
+            q.bits[0] = p.bits[pass];
+        }
+        q.z_base = pass * ksplit;
+        q.ztotal = passes * ksplit;
+        const int lds = plan_lds(q, shape);
+        FLUTE_REQUIRE(lds <= kLdsPerCU, FLUTE_ERR_UNSUPPORTED,
+                      "flute_gemm: %d bytes of LDS exceed the %d of one CU", lds, kLdsPerCU);
+        st = w->lut_dtype == FLUTE_BF16 ? launch_gemm_shape<true>(shape, q, grid, lds, stream)
+                                        : launch_gemm_shape<false>(shape, q, grid, lds, stream);
+        if (st != FLUTE_OK) return st;
+    }
+    return FLUTE_OK;
 }

@@ -55,6 +55,8 @@ struct GemmParams {
     int mblk_total;        // ceil(M / 16)
     int mblk_pad;          // blocks Ap holds per half tile: gridDim.y * MW * MB
     int ksplit, gper;      // gridDim.z and k-tiles per z slice
+    int z_base, ztotal;    // partial tiles: this launch writes [z_base, z_base + gridDim.z) of
+                           // ztotal (several launches, one per stream, may share a fold)
     int out_bf16;          // dtype of C, resA, bias
     int vec_store;         // C rows allow 16-byte stores
 #ifdef FLUTE_GEMM_TRACE
@@ -533,9 +535,9 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     const int unit = blockIdx.y * gridDim.x + blockIdx.x;           // (m chunk, n tile)
     const size_t image = (size_t)ROWS * 128;                        // floats per unit per z
     const size_t zstride = (size_t)gridDim.x * gridDim.y * image;
-    if (p.ksplit > 1) {
+    if (p.ztotal > 1) {
         // across workgroups: partial tiles + ticket; the last arrival folds them in z order
-        float *mine = p.P + (size_t)z * zstride + (size_t)unit * image;
+        float *mine = p.P + (size_t)(p.z_base + z) * zstride + (size_t)unit * image;
         for (int idx = tid; idx < PIECES; idx += NT) {
             const int ml = idx >> 4, n8 = idx & 15;
             ws_store16(mine + ml * 128 + n8 * 8, *(const f4_t *)(tile + ml * LDT + n8 * 8));
@@ -548,7 +550,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         if (tid == 0) {
             const int old = __hip_atomic_fetch_add(p.tickets + unit, 1, __ATOMIC_RELAXED,
                                                    __HIP_MEMORY_SCOPE_AGENT);
-            *flag = (old == p.ksplit - 1);
+            *flag = (old == p.ztotal - 1);
         }
         __syncthreads();
         if (!*flag) return;
@@ -563,13 +565,13 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         if (m >= p.M) continue;
         const int n0 = t * 128 + n8 * 8;
         float y[8];
-        if (p.ksplit > 1) {
+        if (p.ztotal > 1) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) y[e] = 0.0f;
             const float *src = p.P + (size_t)unit * image + ml * 128 + n8 * 8;
-            for (int z0 = 0; z0 < p.ksplit; z0 += 2) {
+            for (int z0 = 0; z0 < p.ztotal; z0 += 2) {
                 const float *s0 = src + z0 * zstride;
-                const float *s1 = z0 + 1 < p.ksplit ? s0 + zstride : s0;
+                const float *s1 = z0 + 1 < p.ztotal ? s0 + zstride : s0;
                 f4_t a, b, c, d;
                 ws_load16x4(s0, s0 + 4, s1, s1 + 4, a, b, c, d);
 #pragma unroll
@@ -577,7 +579,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     y[e] += a[e];
                     y[4 + e] += b[e];
                 }
-                if (z0 + 1 < p.ksplit) {
+                if (z0 + 1 < p.ztotal) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         y[e] += c[e];
