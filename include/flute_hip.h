@@ -174,6 +174,19 @@ flute_status flute_fht(const void *x, const float *signs, const float *awq,
                        void *stream);
 
 /*
+ * Embedding rows out of a palettized table:  out[i, :] = row ids[i] of the table, in
+ * lut_dtype.  Replaces PalettizedEmbedding.forward (scripts/palettized_modules.py:
+ * 1998-2015, 2298-2335), which upstream runs as torch gathers: stream 1 and stream 2
+ * are added in the LUT's 16-bit type (stream 1 first), the residual resA[n, :] @ resB
+ * (both in lut_dtype here) is added in fp32, a rotated (tied) table is un-rotated with
+ * the adjoint transform when w->signs is set, and the row is rounded once.
+ * ids: `count` int64 on the device; an id outside [0, N) yields a row of zeros (the
+ * Python mirror refuses such ids before the launch).  No bias, no awq.
+ */
+flute_status flute_embedding(const flute_linear *w, const int64_t *ids, int64_t count,
+                             void *out, void *stream);
+
+/*
  * The K-split the library would choose for an (N, K) GEMV on this device
  * (the MI355X restatement of gemv_pick_split, src/gemv_host.cpp:29-38).
  * Pure host arithmetic: usable without a GPU.

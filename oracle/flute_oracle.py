@@ -388,3 +388,23 @@ def pick_split_upstream(tiles: int, G: int) -> int:
             break
         s <<= 1
     return best
+
+
+def embedding_reference(ids, blob, lut, N, K, group_size, bits, blob2=None, lut2=None, bits2=0,
+                        resA=None, resB=None, signs=None):
+    """Rows `ids` of a palettized embedding table, in the dtype ladder of
+    PalettizedEmbedding.forward (scripts/palettized_modules.py:1998-2015, 2298-2335):
+    16-bit add of the two streams (stream 1 first), fp32 residual resA[ids] @ resB,
+    adjoint rotation of the sum for a rotated table, one cast to the LUT's dtype.
+    A composition of dequant and fht_adjoint_reference, which carry the pins."""
+    ids = torch.as_tensor(ids).long()
+    w = dequant(blob, lut, N, K, group_size, bits).to(lut.dtype)[ids]
+    if bits2:
+        w = w + dequant(blob2, lut2, N, K, group_size, bits2).to(lut.dtype)[ids]
+    w = w.float()
+    if resA is not None:
+        w = w + resA[ids].float() @ resB.float()
+    if signs is not None:
+        flat = fht_adjoint_reference(w.reshape(-1, K), signs)
+        w = flat.reshape(w.shape)
+    return w.to(lut.dtype)

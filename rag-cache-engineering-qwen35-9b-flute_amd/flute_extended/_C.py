@@ -506,3 +506,35 @@ def gemv_lds_bytes(N: int, K: int, bitwidth: int, bitwidth2: int, group_size: in
     w.lut_rows = (w.N + w.group_size - 1) // w.group_size if w.group_size > 0 else 0
     w.lut_dtype = _lib.F16
     return int(lib.flute_gemv_lds_bytes(ctypes.byref(w), int(split)))
+
+
+def embedding_gather(ids, indices, lut, N: int, K: int, bitwidth: int, group_size: int,
+                     indices2=None, lut2=None, bitwidth2: int = 0, resB=None, resA=None,
+                     signs=None, rot_block: int = 0):
+    """Rows `ids` of a palettized table in the LUT's dtype (PalettizedEmbedding.forward,
+    scripts/palettized_modules.py:2298-2335 upstream).  ids: any integer tensor on the
+    table's device; ids outside [0, N) raise, as upstream's range check does."""
+    who = "embedding_gather"
+    if ids.dtype not in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8):
+        _fail(f"{who}: ids must be an integer tensor, got dtype {ids.dtype}")
+    if ids.device != lut.device:
+        _fail(f"{who}: ids are on {ids.device}, the table on {lut.device}")
+    A = torch.empty((1, int(K)), dtype=lut.dtype, device=lut.device)
+    e8 = _empty_like_u8(A)
+    e16 = torch.empty(0, dtype=A.dtype, device=A.device)
+    w, N2, keep = _describe(who, A, int(K), indices, lut, bitwidth,
+                            indices2 if indices2 is not None else e8,
+                            lut2 if lut2 is not None else e16, bitwidth2,
+                            resB if resB is not None else e16, resA if resA is not None else e16,
+                            e16, group_size, signs, None, rot_block)
+    if N2 != int(N):
+        _fail(f"{who}: blob holds N={N2}, not {N}")
+    flat = ids.reshape(-1).long().contiguous()
+    if flat.numel() and (int(flat.min()) < 0 or int(flat.max()) >= N2):
+        _fail(f"{who}: ids must lie in [0, {N2}) (got min {int(flat.min())}, max {int(flat.max())})")
+    with torch.cuda.device(A.device):
+        out = torch.empty((flat.numel(), int(K)), dtype=lut.dtype, device=lut.device)
+        check(lib.flute_embedding(ctypes.byref(w), flat.data_ptr(), flat.numel(), out.data_ptr(),
+                                  _stream_of(A)))
+    del keep
+    return out.reshape(*ids.shape, int(K))

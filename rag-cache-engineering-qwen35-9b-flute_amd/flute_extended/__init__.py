@@ -44,6 +44,7 @@ from ._C import qgemm_gemv_splitk_fht_stream as _qgemm_gemv_splitk_fht_stream
 from ._C import qgemm_gemv_multi as _qgemm_gemv_multi
 from ._C import qgemm_gemv_mlp as _qgemm_gemv_mlp
 from ._C import dequant_idxn
+from ._C import embedding_gather
 
 Backend = Literal["debug_simple", "cutlass_dense", "cutlass_streaming", "auto"]
 IndicesLayout = Literal["idx1", "idx2", "idx3", "idx4"]
@@ -374,5 +375,5 @@ __all__ = [
     "gemv_splitk_fht_supported", "qgemm_gemv_multi", "gemv_multi_available",
     "gemv_multi_supported", "qgemm_gemv_mlp", "gemv_mlp_available", "gemv_mlp_supported",
     "gemv_split_hint", "GEMV_SPLITK_PAIRS", "GEMV_SPLITK_GROUP_SIZES",
-    "GEMV_SPLITK_MAX_RESIDUAL_RANK", "dequant_idxn",
+    "GEMV_SPLITK_MAX_RESIDUAL_RANK", "dequant_idxn", "embedding_gather",
 ]

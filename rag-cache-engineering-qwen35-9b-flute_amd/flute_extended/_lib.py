@@ -62,6 +62,7 @@ SYMBOLS = {
     "flute_gemm": (_I, [_LP, _P, _P, _I, ctypes.c_int64, ctypes.c_int64, _I, _P]),
     "flute_dequant": (_I, [_LP, _I, _P, _P]),
     "flute_fht": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "flute_embedding": (_I, [_LP, _P, ctypes.c_int64, _P, _P]),
     "flute_pick_split": (_I, [_I, _I]),
     "flute_gemv_lds_bytes": (ctypes.c_int64, [_LP, _I]),
     "flute_validate": (_I, [_LP, _I]),

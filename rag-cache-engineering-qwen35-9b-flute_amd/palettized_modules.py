@@ -573,6 +573,117 @@ class SplitQKV(nn.Module):
         return state
 
 
+class PalettizedEmbedding(nn.Module):
+    """Embedding whose table is a palettized weight: a row gather through the idxN
+    layout (upstream :1979-2335).  Dtype ladder of the module: the two streams are
+    added in the LUT's 16-bit type (stream 1 first), the residual resA[ids] @ resB is
+    added in fp32, a rotated (tied) table is un-rotated with the adjoint transform, and
+    the row is rounded once to the LUT's dtype.  No bias.
+
+    reference=True: torch gathers on any device (upstream's only path).
+    reference=False: one HIP gather launch (flute_embedding) for ids on the GPU."""
+
+    def __init__(self, indices, lut, bitwidth, group_size, N, K, indices2=None, lut2=None,
+                 bitwidth2=None, resA=None, resB=None, num_embeddings=None, embedding_dim=None,
+                 rotation_seed: int = None, rotation_k: int = None, reference: bool = True):
+        super().__init__()
+        self.bitwidth = int(bitwidth)
+        self.bitwidth2 = int(bitwidth2) if bitwidth2 is not None else self.bitwidth
+        for b in (self.bitwidth, self.bitwidth2):
+            if b not in (1, 2, 3, 4):
+                raise ValueError(f"PalettizedEmbedding: bitwidth {b} not in 1..4")
+        self.group_size, self.N, self.K = int(group_size), int(N), int(K)
+        self.reference = bool(reference)
+        if num_embeddings is not None and int(num_embeddings) != self.N:
+            raise ValueError(f"PalettizedEmbedding: num_embeddings {num_embeddings} != N {self.N}")
+        if embedding_dim is not None and int(embedding_dim) != self.K:
+            raise ValueError(f"PalettizedEmbedding: embedding_dim {embedding_dim} != K {self.K}")
+        if self.N % 128 or self.K % 64:
+            raise ValueError(f"idxN layout requires N%128==0 and K%64==0, got N={self.N}, "
+                             f"K={self.K}")
+        if indices.numel() != self.N * self.K * self.bitwidth // 8:
+            raise ValueError(f"idx{self.bitwidth} blob numel {indices.numel()} != "
+                             f"N*K*{self.bitwidth}/8 (N={self.N}, K={self.K})")
+        lut = lut if lut.dim() == 2 else lut.view(-1, 1 << self.bitwidth)
+        if lut.shape[1] != 1 << self.bitwidth:
+            raise ValueError(f"PalettizedEmbedding: LUT palette width {lut.shape[1]} != "
+                             f"2**bitwidth {1 << self.bitwidth}")
+        self.register_buffer("indices", indices, persistent=False)
+        self.register_buffer("lut", lut, persistent=False)
+        if (indices2 is None) != (lut2 is None):
+            raise ValueError("PalettizedEmbedding: a second stream needs BOTH indices2 and lut2")
+        self.has_stream2 = indices2 is not None
+        if self.has_stream2:
+            if indices2.numel() != self.N * self.K * self.bitwidth2 // 8:
+                raise ValueError(f"idx{self.bitwidth2} stream-2 blob numel {indices2.numel()} != "
+                                 f"N*K*{self.bitwidth2}/8")
+            lut2 = lut2 if lut2.dim() == 2 else lut2.view(-1, 1 << self.bitwidth2)
+            if lut2.shape[1] != 1 << self.bitwidth2 or lut2.shape[0] != lut.shape[0]:
+                raise ValueError("PalettizedEmbedding: stream-2 LUT must be "
+                                 f"[{lut.shape[0]}, {1 << self.bitwidth2}], got {tuple(lut2.shape)}")
+            self.register_buffer("indices2", indices2, persistent=False)
+            self.register_buffer("lut2", lut2, persistent=False)
+        else:
+            self.indices2 = self.lut2 = None
+        if resA is not None and resB is not None:
+            if resA.shape != (self.N, resB.shape[0]) or resB.shape[1] != self.K:
+                raise ValueError(f"residual factors shape mismatch: A {tuple(resA.shape)}, B "
+                                 f"{tuple(resB.shape)} for N={self.N}, K={self.K}")
+            self.register_buffer("resA", resA, persistent=False)
+            self.register_buffer("resB", resB, persistent=False)
+        else:
+            self.resA = self.resB = None
+        self.rot_signs = None
+        if rotation_seed is not None and rotation_k is not None:
+            if int(rotation_k) != self.K:
+                raise ValueError(f"PalettizedEmbedding: rotation_k {rotation_k} != K {self.K}")
+            self.rot_signs = _get_fht().rotation_signs(self.K, int(rotation_seed))
+        self._logical = {}
+
+    num_embeddings = property(lambda self: self.N)
+    embedding_dim = property(lambda self: self.K)
+
+    def _logical_indices(self, which):
+        key = (which, self.indices.device)
+        if key not in self._logical:
+            blob = self.indices if which == 1 else self.indices2
+            bits = self.bitwidth if which == 1 else self.bitwidth2
+            idx = _get_idxn().unpack_idxn(blob.cpu().numpy(), self.N, self.K, bits)
+            self._logical[key] = torch.from_numpy(idx).to(blob.device)
+        return self._logical[key]
+
+    def _gather_stream(self, ids, lut, which):
+        rows = lut[torch.clamp(ids // self.group_size, max=lut.shape[0] - 1)]
+        return rows.gather(-1, self._logical_indices(which)[ids].long())
+
+    def forward(self, ids):
+        if not torch.is_tensor(ids):
+            ids = torch.as_tensor(ids)
+        if ids.dtype not in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8):
+            raise ValueError(f"PalettizedEmbedding.forward: ids must be an integer tensor, got "
+                             f"dtype {ids.dtype}")
+        ids = ids.long()
+        if ids.numel() and (int(ids.min()) < 0 or int(ids.max()) >= self.N):
+            raise ValueError(f"PalettizedEmbedding.forward: ids must lie in [0, {self.N})")
+        if not self.reference and ids.is_cuda:
+            _count("embedding_gather")
+            signs = None if self.rot_signs is None else self.rot_signs.to(ids.device)
+            return _flute().embedding_gather(
+                ids, self.indices, self.lut, self.N, self.K, self.bitwidth, self.group_size,
+                indices2=self.indices2, lut2=self.lut2,
+                bitwidth2=self.bitwidth2 if self.has_stream2 else 0,
+                resB=self.resB, resA=self.resA, signs=signs)
+        w = self._gather_stream(ids, self.lut, 1)
+        if self.has_stream2:
+            w = w + self._gather_stream(ids, self.lut2, 2)
+        w = w.float()
+        if self.resA is not None:
+            w = w + self.resA[ids].float() @ self.resB.float()
+        if self.rot_signs is not None:
+            w = _get_fht().fht_adjoint(w, self.rot_signs.to(w.device), backend="reference")
+        return w.to(self.lut.dtype)
+
+
 def act_name(fn) -> str:
     name = getattr(fn, "__name__", None) or type(fn).__name__
     return name.lower().replace("activation", "")
