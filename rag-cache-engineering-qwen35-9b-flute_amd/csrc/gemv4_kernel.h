@@ -25,6 +25,10 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
     constexpr int SPT = 128 / RW;                   // row slices per tile
     constexpr int PF = NW == 4 ? 8 : 4;             // wavefront loads in flight per lane
     constexpr int XV = 2;                           // 16-byte activation loads per thread
+#ifndef FLUTE_GEMV4_LB
+#define FLUTE_GEMV4_LB 4
+#endif
+    constexpr int LB = FLUTE_GEMV4_LB;              // dwords of a load looked up per batch
     constexpr int STRIDE = 1 << ES;                 // table bytes per entry
     constexpr int CHUNKS = STRIDE / 16;             // 16-byte pieces of one entry's replicas
     constexpr int SHARES = NT / 256;                // threads per table entry
@@ -156,27 +160,40 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
                 for (int n = 0; n < PF; ++n) {
                     const int m = nb + n;
                     if (m < my_units) {             // uniform within the wavefront
-                        const uint32_t wq[4] = {q[n].x, q[n].y, q[n].z, q[n].w};
-                        if (m + PF < my_units)
-                            q[n] = *(const uint4 *)(qrow + (lane0 + (uint32_t)(m + PF) * step));
                         const int xo = xi + m * (NW * GPI * 32);
                         const uint32_t xa = xs32[xo];
                         const uint32_t xb = xs32[xo + 4];
+                        // The lookups of LB dwords of the load go out together and are
+                        // consumed together, so their LDS latency is paid once per batch,
+                        // not once per dword.
 #pragma unroll
-                        for (int v = 0; v < 4; ++v) {
+                        for (int vb = 0; vb < 4; vb += LB) {
+                            uint32_t e[LB][4];
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) {   // byte j: d = j >> 1, s2 = j & 1
-                                uint32_t addr;
-                                if constexpr (ES == 8) {
-                                    addr = __builtin_amdgcn_perm(wq[v], slot,
-                                                                 0x03020000u | ((4u + j) << 8));
-                                } else {
-                                    addr = (((wq[v] >> (8 * j)) & 0xffu) << ES) + slot;
+                            for (int v = 0; v < LB; ++v) {
+                                const uint32_t wv = vb + v == 0 ? q[n].x
+                                                  : vb + v == 1 ? q[n].y
+                                                  : vb + v == 2 ? q[n].z : q[n].w;
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {   // byte j: d = j >> 1, s2 = j & 1
+                                    uint32_t addr;
+                                    if constexpr (ES == 8) {
+                                        addr = __builtin_amdgcn_perm(wv, slot,
+                                                                     0x03020000u | ((4u + j) << 8));
+                                    } else {
+                                        addr = (((wv >> (8 * j)) & 0xffu) << ES) + slot;
+                                    }
+                                    e[v][j] = *(LdsWord)addr;
                                 }
-                                const uint32_t e = *(LdsWord)addr;
-                                acc[v * 2 + (j >> 1)] =
-                                    dot2<BF16>(e, (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
                             }
+                            if (vb + LB == 4 && m + PF < my_units)   // indices consumed: refill
+                                q[n] = *(const uint4 *)(qrow + (lane0 + (uint32_t)(m + PF) * step));
+#pragma unroll
+                            for (int v = 0; v < LB; ++v)
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+                                    acc[(vb + v) * 2 + (j >> 1)] = dot2<BF16>(
+                                        e[v][j], (j & 1) ? xb : xa, acc[(vb + v) * 2 + (j >> 1)]);
                         }
                     }
                 }
