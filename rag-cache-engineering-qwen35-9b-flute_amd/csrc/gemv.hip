@@ -83,9 +83,12 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
     int wv = env_int("FLUTE_GEMV_WAVES", 0);
     if (wv != 1 && wv != 2 && wv != 4 && wv != 8) {
         // four wavefronts with eight loads each in flight measured best; eight when a
-        // workgroup has a long K range to itself
+        // workgroup has a long K range to itself and the grid is small enough for all
+        // of it to be resident at once with eight (two workgroups per CU)
         const int units = (G / sp) / (32 / best_rw);
-        wv = units >= 64 ? 8 : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
+        const long wgs = (long)(rows / best_rw) * sp;
+        wv = (units >= 64 && wgs <= 2 * kNumCU) ? 8
+                                                : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
     }
     *waves = wv;
 }

@@ -16,7 +16,10 @@ namespace flute {
 // MULTI = several independent weights share the launch (the descriptor is then
 //         picked by grid column, which costs a dependent scalar load).
 template <int LPGL, int NW, int ES, bool BF16, bool MULTI>
-__global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
+// Three wavefronts per SIMD (168 registers), except where the 64 KB table already
+// limits a CU to two four-wavefront workgroups.
+__global__ void __launch_bounds__(NW * 64, (NW == 4 && ES == 8) ? 2 : 3)
+    gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int NT = NW * 64;
     constexpr int LPG = 1 << LPGL;
@@ -25,10 +28,10 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
     constexpr int SPT = 128 / RW;                   // row slices per tile
     constexpr int PF = NW == 4 ? 8 : 4;             // wavefront loads in flight per lane
     constexpr int XV = 2;                           // 16-byte activation loads per thread
-#ifndef FLUTE_GEMV4_LB
-#define FLUTE_GEMV4_LB 4
+#ifndef FLUTE_GEMV4_PF0
+#define FLUTE_GEMV4_PF0 2
 #endif
-    constexpr int LB = FLUTE_GEMV4_LB;              // dwords of a load looked up per batch
+    constexpr int PF0 = FLUTE_GEMV4_PF0 < PF ? FLUTE_GEMV4_PF0 : PF;   // index loads ahead of the table
     constexpr int STRIDE = 1 << ES;                 // table bytes per entry
     constexpr int CHUNKS = STRIDE / 16;             // 16-byte pieces of one entry's replicas
     constexpr int SHARES = NT / 256;                // threads per table entry
@@ -36,6 +39,7 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
     static_assert(NT >= 256, "one thread per table entry at least");
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
+    warm_kernargs<(int)sizeof(GemvParams)>(kp);
     int si0 = 0;
     if (MULTI && !p.silu_mul) {
 #pragma unroll
@@ -78,142 +82,282 @@ __global__ void __launch_bounds__(NW * 64) gemv4_kernel(const GemvParams p) {
     const int share = tid >> 8;
 
     const int nout = p.silu_mul ? 2 : 1;
-    const uint16_t *staged_x = nullptr;
-    const float *staged_signs = nullptr, *staged_awq = nullptr;
-    bool staged = false;
+
+    // A pass is one (output, stream) of this workgroup's rows: one output with one
+    // stream for a plain weight, two streams for a dual-stream weight, two outputs
+    // for the gate/up pair.  Every pass covers the same K range with the same lane
+    // geometry; only the index blob and the LUT row change.
+    auto pass_ptrs = [&](int so_, int si_, const uint8_t *&qr, const uint16_t *&lutp) {
+        const int sg = so_ == 1 ? 1 : si0;
+        const GemvStream st = kp->seg[sg].st[si_];
+        const int grp = min((t * 128) >> __builtin_ctz(kp->seg[sg].gs), kp->seg[sg].lut_rows - 1);
+        qr = st.q + ((size_t)t * G + g_lo) * 4096u;
+        lutp = st.lut + ((size_t)grp << 4);
+    };
+    // A wavefront with fewer than PF loads re-reads the first unit of the K range
+    // (always present) into the registers it will not consume: every load below is
+    // unconditional, so the compiler knows how many are in flight at each point and
+    // waits for exactly the one it needs.  One conditional load in a loop makes it
+    // wait for all of them at the loop head, which serialises the memory stream and
+    // the arithmetic.
+    // Index loads are addressed as (uniform base + unit offset) in scalar registers
+    // plus one lane-constant 32-bit offset, so no per-load address lives in vector
+    // registers.
+    auto unit_load = [&](const uint8_t *qr, int unit) -> uint4 {
+        const uint8_t *base = unit < my_units ? qr + (size_t)unit * step
+                                              : qr - (size_t)w * unit_bytes;
+        return *(const uint4 *)(base + lane0);
+    };
+    auto first_units = [&](const uint8_t *qr, uint4 (&qq)[PF]) {
+#pragma unroll
+        for (int n = 0; n < PF; ++n) {
+            qq[n] = unit_load(qr, n);
+            __builtin_amdgcn_sched_barrier(0);      // issue order = consumption order
+        }
+    };
+
+    // Paired table: entry e -> {lut[e & 15], lut[e >> 4]}, replicated over the stride;
+    // 16 bytes per store, starting at a lane-dependent piece so that a wavefront
+    // spreads over the banks.
+    auto write_table = [&](uint32_t lo_, uint32_t hi_) {
+        const uint32_t v = lo_ | (hi_ << 16);
+        const uint4 v4 = make_uint4(v, v, v, v);
+        uint8_t *ent = lds + e_own * STRIDE + share * (CPT * 16);
+#pragma unroll
+        for (int k = 0; k < CPT; ++k) *(uint4 *)(ent + (((k + tid) & (CPT - 1)) << 4)) = v4;
+    };
 
     FLUTE_TRACE(0);
-    for (int so = 0; so < nout; ++so) {
-        const int si_seg = so == 1 ? 1 : si0;
-        const uint16_t *xin = kp->seg[si_seg].xsrc ? kp->seg[si_seg].xsrc : p.x;
-        const float *signs = kp->seg[si_seg].signs, *awq = kp->seg[si_seg].awq;
-        const int nstreams = kp->seg[si_seg].nstreams;
-        const int lut_rows = kp->seg[si_seg].lut_rows;
-        const int grp = min((t * 128) / kp->seg[si_seg].gs, lut_rows - 1);
-        const bool restage = !staged || xin != staged_x || signs != staged_signs || awq != staged_awq;
-        const bool x_direct = restage && signs == nullptr;     // plain copy: loads issued first
-
-        float acc[8];
+    // ---- first pass: activations, LUT values and the first index bytes.  The order
+    //      of the loads is the order they are needed in, and the scheduler is kept
+    //      from changing it: a wait for an early load also waits for everything
+    //      issued before it. ---------------------------------------------------------
+    int so = 0, si = 0;
+    const uint8_t *qrow;
+    const uint16_t *lut;
+    pass_ptrs(0, 0, qrow, lut);
+    const uint16_t *staged_x = kp->seg[si0].xsrc ? kp->seg[si0].xsrc : p.x;
+    const float *staged_signs = kp->seg[si0].signs, *staged_awq = kp->seg[si0].awq;
+    const bool x_direct = staged_signs == nullptr;  // plain copy
+    const bool x_short = kc <= XV * NT * 8;         // uniform
+    uint4 q[PF];
+    uint32_t lo, hi;
+    if (x_direct && x_short) {
+        // The usual case.  A few index loads go out ahead of the table build so that
+        // the memory stream starts early; the rest follow once the table is written.
+        // (All of them at once would put every other workgroup's activation and LUT
+        // loads behind a full batch of index bytes in the CU's memory queue.)
+        uint4 xv[XV];
 #pragma unroll
-        for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
-
-        for (int si = 0; si < nstreams; ++si) {
-            const GemvStream st = kp->seg[si_seg].st[si];
-            // ---- loads, in the order they are needed: activations, LUT, indices ----
-            uint4 xv[XV];
-            if (si == 0 && x_direct) {
+        for (int i = 0; i < XV; ++i) {
+            const int j = (i * NT + tid) * 8;
+            xv[i] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        lo = lut[e_own & 15];
+        hi = lut[e_own >> 4];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int i = 0; i < XV; ++i) {
-                    const int j = (i * NT + tid) * 8;
-                    xv[i] = make_uint4(0u, 0u, 0u, 0u);
-                    if (j < kc) xv[i] = *(const uint4 *)(xin + k0 + j);
-                }
-            }
-            const uint16_t *lut = st.lut + ((size_t)grp << 4);
-            const uint32_t lo = lut[e_own & 15], hi = lut[e_own >> 4];
-            const uint8_t *qrow = st.q + ((size_t)t * G + g_lo) * 4096u;
-            uint4 q[PF];
+        for (int n = 0; n < PF0; ++n) {
+            q[n] = unit_load(qrow, n);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        FLUTE_TRACE(1);
+#pragma unroll
+        for (int i = 0; i < XV; ++i) {
+            const int j = (i * NT + tid) * 8;
+            if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(xv[i], p.act_bf16);
+        }
+        write_table(lo, hi);
+#pragma unroll
+        for (int n = PF0; n < PF; ++n) {
+            q[n] = unit_load(qrow, n);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        // A long K range, or a rotated input: everything the table and the staged
+        // activations need is fetched and written first (the index registers carry the
+        // activations meanwhile), then the index loads start.
+        if (x_direct) {
 #pragma unroll
             for (int n = 0; n < PF; ++n) {
-                q[n] = make_uint4(0u, 0u, 0u, 0u);
-                if (n < my_units) q[n] = *(const uint4 *)(qrow + (lane0 + (uint32_t)n * step));
+                const int j = (n * NT + tid) * 8;
+                q[n] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
             }
-
-            FLUTE_TRACE(1);
-            // ---- activations into LDS ---------------------------------------------
-            if (si == 0 && restage) {
-                if (x_direct) {
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        lo = lut[e_own & 15];
+        hi = lut[e_own >> 4];
+        __builtin_amdgcn_sched_barrier(0);
+        FLUTE_TRACE(1);
+        if (x_direct) {
 #pragma unroll
-                    for (int i = 0; i < XV; ++i) {
-                        const int j = (i * NT + tid) * 8;
-                        if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(xv[i], p.act_bf16);
-                    }
-                    for (int j = (XV * NT + tid) * 8; j < kc; j += NT * 8)
-                        *(uint4 *)(xs + j) =
-                            to_compute_type<BF16>(*(const uint4 *)(xin + k0 + j), p.act_bf16);
-                } else {
+            for (int n = 0; n < PF; ++n) {
+                const int j = (n * NT + tid) * 8;
+                if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(q[n], p.act_bf16);
+            }
+            for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8)
+                *(uint4 *)(xs + j) =
+                    to_compute_type<BF16>(*(const uint4 *)(staged_x + k0 + j), p.act_bf16);
+        } else {
+            stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
+        }
+        write_table(lo, hi);
+        __builtin_amdgcn_sched_barrier(0);
+        first_units(qrow, q);
+    }
+
+    float acc[8];
+#pragma unroll
+    for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
+
+    for (bool first = true;; first = false) {
+        const int sg = so == 1 ? 1 : si0;
+        if (!first) {
+            if (si == 0) {                          // a new output: restage if its input differs
+                const uint16_t *xin = kp->seg[sg].xsrc ? kp->seg[sg].xsrc : p.x;
+                const float *signs = kp->seg[sg].signs, *awq = kp->seg[sg].awq;
+                if (xin != staged_x || signs != staged_signs || awq != staged_awq) {
                     stage_x<BF16>(p, xin, signs, awq, lds, k0, kc, tid, NT);
+                    staged_x = xin;
+                    staged_signs = signs;
+                    staged_awq = awq;
                 }
-                staged = true;
-                staged_x = xin;
-                staged_signs = signs;
-                staged_awq = awq;
             }
+            write_table(lo, hi);
+        }
 
-            // ---- paired table: entry e -> {lut[e & 15], lut[e >> 4]}, replicated over
-            //      the stride; 16 bytes per store, starting at a lane-dependent piece so
-            //      that a wavefront spreads over the banks --------------------------------
-            {
-                const uint32_t v = lo | (hi << 16);
-                const uint4 v4 = make_uint4(v, v, v, v);
-                uint8_t *ent = lds + e_own * STRIDE + share * (CPT * 16);
+        // ---- the pass after this one: its LUT values are fetched now and its first
+        //      index loads replace this pass's last ones as they are consumed, so the
+        //      memory stream does not stop between passes.  Without a next pass the
+        //      same LUT values are read again (harmless, and keeps the load count
+        //      unconditional). -----------------------------------------------------------
+        int nso = so, nsi = si + 1;
+        if (nsi == kp->seg[sg].nstreams) {
+            nsi = 0;
+            nso = so + 1;
+        }
+        const bool has_next = nso < nout;
+        const uint8_t *qnext = qrow;
+        const uint16_t *lutn = lut;
+        if (has_next) pass_ptrs(nso, nsi, qnext, lutn);
+        __builtin_amdgcn_sched_barrier(0);
+        lo = lutn[e_own & 15];
+        hi = lutn[e_own >> 4];
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+#ifdef FLUTE_GEMV_TRACE
+        if (first) FLUTE_TRACE(2); else if (so == 1 && si == 0) FLUTE_TRACE(7);
+#endif
+
+        // ---- K loop -----------------------------------------------------------------
+        // One unit = one 16-byte load of this lane.  Its sixteen table lookups go out
+        // together and are consumed together, so the LDS latency is paid once per
+        // load, not once per dword.
+        auto lookups = [&](const uint4 &qv, uint32_t (&e)[4][4]) {
 #pragma unroll
-                for (int k = 0; k < CPT; ++k)
-                    *(uint4 *)(ent + (((k + tid) & (CPT - 1)) << 4)) = v4;
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t wv = v == 0 ? qv.x : v == 1 ? qv.y : v == 2 ? qv.z : qv.w;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {       // byte j: d = j >> 1, s2 = j & 1
+                    uint32_t addr;
+                    if constexpr (ES == 8) {
+                        addr = __builtin_amdgcn_perm(wv, slot, 0x03020000u | ((4u + j) << 8));
+                    } else {
+                        addr = (((wv >> (8 * j)) & 0xffu) << ES) + slot;
+                    }
+                    e[v][j] = *(LdsWord)addr;
+                }
             }
-            __syncthreads();
-            FLUTE_TRACE(2);
-
-            // ---- K loop -----------------------------------------------------------
-            for (int nb = 0; nb < my_units; nb += PF) {
+        };
+        auto dots = [&](const uint32_t (&e)[4][4], int m) {
+            const int xo = xi + m * (NW * GPI * 32);
+            const uint32_t xa = xs32[xo];
+            const uint32_t xb = xs32[xo + 4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[v * 2 + (j >> 1)] =
+                        dot2<BF16>(e[v][j], (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
+        };
+        int nb = 0;
+        for (; nb + 2 * PF <= my_units; nb += PF) {          // every refill exists
+#pragma unroll
+            for (int n = 0; n < PF; ++n) {
+                uint32_t e[4][4];
+                lookups(q[n], e);
+                // pinned: the scheduler would otherwise sink all refills to the end of
+                // the body, draining the prefetch queue once per group
+                __builtin_amdgcn_sched_barrier(0);
+                q[n] = *(const uint4 *)(qrow + (size_t)(nb + n + PF) * step + lane0);
+                __builtin_amdgcn_sched_barrier(0);
+                dots(e, nb + n);
+            }
+        }
+        if (nb + PF == my_units && has_next) {                // a full last group, refilled
+#pragma unroll                                                //   from the next pass
+            for (int n = 0; n < PF; ++n) {
+                uint32_t e[4][4];
+                lookups(q[n], e);
+                __builtin_amdgcn_sched_barrier(0);
+                q[n] = *(const uint4 *)(qnext + (size_t)n * step + lane0);
+                __builtin_amdgcn_sched_barrier(0);
+                dots(e, nb + n);
+            }
+        } else if (nb + PF >= my_units) {                     // the last group, no refills
+#pragma unroll
+            for (int n = 0; n < PF; ++n) {
+                if (nb + n < my_units) {                      // uniform within the wavefront
+                    uint32_t e[4][4];
+                    lookups(q[n], e);
+                    dots(e, nb + n);
+                }
+            }
+            if (has_next) first_units(qnext, q);
+        } else {                                              // a partial group follows
+            for (; nb < my_units; nb += PF) {
 #pragma unroll
                 for (int n = 0; n < PF; ++n) {
                     const int m = nb + n;
-                    if (m < my_units) {             // uniform within the wavefront
-                        const int xo = xi + m * (NW * GPI * 32);
-                        const uint32_t xa = xs32[xo];
-                        const uint32_t xb = xs32[xo + 4];
-                        // The lookups of LB dwords of the load go out together and are
-                        // consumed together, so their LDS latency is paid once per batch,
-                        // not once per dword.
-#pragma unroll
-                        for (int vb = 0; vb < 4; vb += LB) {
-                            uint32_t e[LB][4];
-#pragma unroll
-                            for (int v = 0; v < LB; ++v) {
-                                const uint32_t wv = vb + v == 0 ? q[n].x
-                                                  : vb + v == 1 ? q[n].y
-                                                  : vb + v == 2 ? q[n].z : q[n].w;
-#pragma unroll
-                                for (int j = 0; j < 4; ++j) {   // byte j: d = j >> 1, s2 = j & 1
-                                    uint32_t addr;
-                                    if constexpr (ES == 8) {
-                                        addr = __builtin_amdgcn_perm(wv, slot,
-                                                                     0x03020000u | ((4u + j) << 8));
-                                    } else {
-                                        addr = (((wv >> (8 * j)) & 0xffu) << ES) + slot;
-                                    }
-                                    e[v][j] = *(LdsWord)addr;
-                                }
-                            }
-                            if (vb + LB == 4 && m + PF < my_units)   // indices consumed: refill
-                                q[n] = *(const uint4 *)(qrow + (lane0 + (uint32_t)(m + PF) * step));
-#pragma unroll
-                            for (int v = 0; v < LB; ++v)
-#pragma unroll
-                                for (int j = 0; j < 4; ++j)
-                                    acc[(vb + v) * 2 + (j >> 1)] = dot2<BF16>(
-                                        e[v][j], (j & 1) ? xb : xa, acc[(vb + v) * 2 + (j >> 1)]);
-                        }
+                    if (m < my_units) {
+                        uint32_t e[4][4];
+                        lookups(q[n], e);
+                        if (m + PF < my_units)
+                            q[n] = *(const uint4 *)(qrow + (size_t)(m + PF) * step + lane0);
+                        dots(e, m);
                     }
                 }
             }
-            FLUTE_TRACE(3);
-            __syncthreads();                       // the table region is rewritten next
+            __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): see below
+            if (has_next) first_units(qnext, q);
         }
+#ifdef FLUTE_GEMV_TRACE
+        if (!has_next) FLUTE_TRACE(3); else if (first) FLUTE_TRACE(6);
+#endif
 
-        // fold the lanes that share rows
+        // ---- end of an output: fold the lanes that share rows ------------------------
+        if (nso != so) {
 #pragma unroll
-        for (int a = 0; a < 8; ++a) {
-            float v = row16_sum(acc[a]);
-            if constexpr (LPGL <= 5) v += __shfl_xor(v, 32);
-            if constexpr (LPGL == 4) v += __shfl_xor(v, 16);
-            acc[a] = v;
-        }
-        if (L < LPG && (L & 15) == 0) {
+            for (int a = 0; a < 8; ++a) {
+                float v = row16_sum(acc[a]);
+                if constexpr (LPGL <= 5) v += __shfl_xor(v, 32);
+                if constexpr (LPGL == 4) v += __shfl_xor(v, 16);
+                acc[a] = v;
+            }
+            if (L < LPG && (L & 15) == 0) {
 #pragma unroll
-            for (int a = 0; a < 8; ++a) red[(so * NW + w) * 32 + (L >> 4) * 8 + a] = acc[a];
+                for (int a = 0; a < 8; ++a) red[(so * NW + w) * 32 + (L >> 4) * 8 + a] = acc[a];
+            }
+#pragma unroll
+            for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
         }
+        if (!has_next) break;
+        __syncthreads();                            // the table region is rewritten next
+        so = nso;
+        si = nsi;
+        qrow = qnext;
+        lut = lutn;
     }
     __syncthreads();
     FLUTE_TRACE(4);

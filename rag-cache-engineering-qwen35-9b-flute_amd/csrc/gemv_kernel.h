@@ -89,6 +89,20 @@ struct GemvParams {
 #endif
 };
 
+// Reads one dword of every 64-byte line of the kernel-argument block with
+// independent scalar loads and waits for them once.  The descriptor fields are
+// then fetched through a chain of dependent scalar loads (segment -> stream ->
+// pointers); with the lines already in the scalar cache each link costs a cache
+// hit instead of a trip to L2 or memory.
+template <int BYTES>
+__device__ __forceinline__ void warm_kernargs(const void *kernargs) {
+    const uint32_t *ka = (const uint32_t *)kernargs;
+    uint32_t seen = 0;
+#pragma unroll
+    for (int o = 0; o < BYTES; o += 64) seen |= ka[o / 4];
+    asm volatile("" ::"s"(seen));
+}
+
 #ifdef FLUTE_GEMV_TRACE
 #define FLUTE_TRACE(slot)                                                              \
     do {                                                                               \
@@ -151,7 +165,10 @@ template <int B, bool BF16, bool PERM>
 __device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t xa, uint32_t xb,
                                                 const uint8_t *lds, const uint32_t (&lane_off)[4],
                                                 int es, float (&acc)[8]) {
+    // Every table lookup of the quarter is issued before the first dot product, so
+    // the LDS latency is paid once per quarter rather than once per lookup.
     if constexpr (B == 4) {
+        uint32_t e[4][4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
 #pragma unroll
@@ -162,11 +179,16 @@ __device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t
                 } else {
                     addr = (((w[v] >> (8 * j)) & 0xffu) << es) + lane_off[v];
                 }
-                const uint32_t e = *(const uint32_t *)(lds + addr);
-                acc[v * 2 + (j >> 1)] = dot2<BF16>(e, (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
+                e[v][j] = *(const uint32_t *)(lds + addr);
             }
         }
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[v * 2 + (j >> 1)] = dot2<BF16>(e[v][j], (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
     } else if constexpr (B == 2) {
+        uint2 e[4][2];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
 #pragma unroll
@@ -179,12 +201,19 @@ __device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t
                 } else {
                     addr = (((w[v >> 1] >> (8 * j)) & 0xffu) << es) + lane_off[v];
                 }
-                const uint2 e = *(const uint2 *)(lds + addr);
-                acc[v * 2 + d] = dot2<BF16>(e.x, xa, acc[v * 2 + d]);
-                acc[v * 2 + d] = dot2<BF16>(e.y, xb, acc[v * 2 + d]);
+                e[v][d] = *(const uint2 *)(lds + addr);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+#pragma unroll
+            for (int d = 0; d < 2; ++d) {
+                acc[v * 2 + d] = dot2<BF16>(e[v][d].x, xa, acc[v * 2 + d]);
+                acc[v * 2 + d] = dot2<BF16>(e[v][d].y, xb, acc[v * 2 + d]);
             }
         }
     } else if constexpr (B == 1) {
+        uint4 e[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {               // byte v of the single dword
             uint32_t addr;
@@ -193,11 +222,14 @@ __device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t
             } else {
                 addr = (((w[0] >> (8 * v)) & 0xffu) << es) + lane_off[v];
             }
-            const uint4 e = *(const uint4 *)(lds + addr);
-            acc[v * 2 + 0] = dot2<BF16>(e.x, xa, acc[v * 2 + 0]);
-            acc[v * 2 + 0] = dot2<BF16>(e.y, xb, acc[v * 2 + 0]);
-            acc[v * 2 + 1] = dot2<BF16>(e.z, xa, acc[v * 2 + 1]);
-            acc[v * 2 + 1] = dot2<BF16>(e.w, xb, acc[v * 2 + 1]);
+            e[v] = *(const uint4 *)(lds + addr);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            acc[v * 2 + 0] = dot2<BF16>(e[v].x, xa, acc[v * 2 + 0]);
+            acc[v * 2 + 0] = dot2<BF16>(e[v].y, xb, acc[v * 2 + 0]);
+            acc[v * 2 + 1] = dot2<BF16>(e[v].z, xa, acc[v * 2 + 1]);
+            acc[v * 2 + 1] = dot2<BF16>(e[v].w, xb, acc[v * 2 + 1]);
         }
     } else {                                        // B == 3: one 24-bit group per v
         const uint32_t grp[4] = {
@@ -206,15 +238,20 @@ __device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t
             __builtin_amdgcn_alignbit(w[2], w[1], 16),
             w[2] >> 8,
         };
+        uint32_t e[4][4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
 #pragma unroll
             for (int f = 0; f < 4; ++f) {          // field f: d = f >> 1, s2 = f & 1
                 const uint32_t code = (grp[v] >> (6 * f)) & 63u;
-                const uint32_t e = *(const uint32_t *)(lds + (code << es) + lane_off[v]);
-                acc[v * 2 + (f >> 1)] = dot2<BF16>(e, (f & 1) ? xb : xa, acc[v * 2 + (f >> 1)]);
+                e[v][f] = *(const uint32_t *)(lds + (code << es) + lane_off[v]);
             }
         }
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+                acc[v * 2 + (f >> 1)] = dot2<BF16>(e[v][f], (f & 1) ? xb : xa, acc[v * 2 + (f >> 1)]);
     }
 }
 
@@ -555,6 +592,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 4) gemv_kernel(const GemvPara
     // (constant address space): a dynamic index then costs a scalar load with an
     // offset instead of a select chain over every field of every descriptor.
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
+    warm_kernargs<(int)sizeof(GemvParams)>(kp);
     int si0 = 0;
     if (!p.silu_mul) {
 #pragma unroll
