@@ -158,78 +158,42 @@ __device__ __forceinline__ uint32_t table_dword(const uint16_t *lut, int e, int 
     return (uint32_t)lut[c0] | ((uint32_t)lut[c1] << 16);
 }
 
-// One quarter-chunk (4*B bytes of this lane) against the activation pairs xa
-// (s2 = 0) and xb (s2 = 1).  lane_off[v] = table base of row block v plus this
-// lane's replica offset.
-template <int B, bool BF16, bool PERM>
-__device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t xa, uint32_t xb,
-                                                const uint8_t *lds, const uint32_t (&lane_off)[4],
-                                                int es, float (&acc)[8]) {
-    // Every table lookup of the quarter is issued before the first dot product, so
-    // the LDS latency is paid once per quarter rather than once per lookup.
+// One quarter-chunk (4*B bytes of this lane) in two steps, so that the refill of
+// the index registers can be issued between them: every table lookup of the
+// quarter goes out first (the LDS latency is paid once per quarter, not once per
+// lookup), then the looked-up pairs meet the activation pairs xa (s2 = 0) and xb
+// (s2 = 1).  lane_off[v] = table base of row block v plus this lane's replica
+// offset.  Whatever the width, a quarter looks up 16 dwords.
+template <int B>
+__device__ __forceinline__ void quarter_lookups(const uint32_t (&w)[B], const uint8_t *lds,
+                                                const uint32_t (&lane_off)[4], int es,
+                                                uint32_t (&e)[16]) {
+    auto byte_addr = [&](uint32_t word, int j, uint32_t off) -> uint32_t {
+        return (((word >> (8 * j)) & 0xffu) << es) + off;
+    };
     if constexpr (B == 4) {
-        uint32_t e[4][4];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {          // byte j: d = j >> 1, s2 = j & 1
-                uint32_t addr;
-                if constexpr (PERM) {
-                    addr = __builtin_amdgcn_perm(w[v], lane_off[v], 0x03020000u | ((4u + j) << 8));
-                } else {
-                    addr = (((w[v] >> (8 * j)) & 0xffu) << es) + lane_off[v];
-                }
-                e[v][j] = *(const uint32_t *)(lds + addr);
-            }
-        }
 #pragma unroll
         for (int v = 0; v < 4; ++v)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[v * 2 + (j >> 1)] = dot2<BF16>(e[v][j], (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
+            for (int j = 0; j < 4; ++j)             // byte j: d = j >> 1, s2 = j & 1
+                e[v * 4 + j] = *(const uint32_t *)(lds + byte_addr(w[v], j, lane_off[v]));
     } else if constexpr (B == 2) {
-        uint2 e[4][2];
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
+        for (int v = 0; v < 4; ++v)
 #pragma unroll
-            for (int d = 0; d < 2; ++d) {
-                const int j = (v & 1) * 2 + d;      // byte j of dword v >> 1
-                uint32_t addr;
-                if constexpr (PERM) {
-                    addr = __builtin_amdgcn_perm(w[v >> 1], lane_off[v],
-                                                 0x03020000u | ((4u + j) << 8));
-                } else {
-                    addr = (((w[v >> 1] >> (8 * j)) & 0xffu) << es) + lane_off[v];
-                }
-                e[v][d] = *(const uint2 *)(lds + addr);
+            for (int d = 0; d < 2; ++d) {           // byte (v & 1) * 2 + d of dword v >> 1
+                const uint2 t = *(const uint2 *)(lds + byte_addr(w[v >> 1], (v & 1) * 2 + d, lane_off[v]));
+                e[(v * 2 + d) * 2] = t.x;
+                e[(v * 2 + d) * 2 + 1] = t.y;
             }
-        }
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-#pragma unroll
-            for (int d = 0; d < 2; ++d) {
-                acc[v * 2 + d] = dot2<BF16>(e[v][d].x, xa, acc[v * 2 + d]);
-                acc[v * 2 + d] = dot2<BF16>(e[v][d].y, xb, acc[v * 2 + d]);
-            }
-        }
     } else if constexpr (B == 1) {
-        uint4 e[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {               // byte v of the single dword
-            uint32_t addr;
-            if constexpr (PERM) {
-                addr = __builtin_amdgcn_perm(w[0], lane_off[v], 0x03020000u | ((4u + v) << 8));
-            } else {
-                addr = (((w[0] >> (8 * v)) & 0xffu) << es) + lane_off[v];
-            }
-            e[v] = *(const uint4 *)(lds + addr);
-        }
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            acc[v * 2 + 0] = dot2<BF16>(e[v].x, xa, acc[v * 2 + 0]);
-            acc[v * 2 + 0] = dot2<BF16>(e[v].y, xb, acc[v * 2 + 0]);
-            acc[v * 2 + 1] = dot2<BF16>(e[v].z, xa, acc[v * 2 + 1]);
-            acc[v * 2 + 1] = dot2<BF16>(e[v].w, xb, acc[v * 2 + 1]);
+            const uint4 t = *(const uint4 *)(lds + byte_addr(w[0], v, lane_off[v]));
+            e[v * 4] = t.x;
+            e[v * 4 + 1] = t.y;
+            e[v * 4 + 2] = t.z;
+            e[v * 4 + 3] = t.w;
         }
     } else {                                        // B == 3: one 24-bit group per v
         const uint32_t grp[4] = {
@@ -238,36 +202,70 @@ __device__ __forceinline__ void consume_quarter(const uint32_t (&w)[B], uint32_t
             __builtin_amdgcn_alignbit(w[2], w[1], 16),
             w[2] >> 8,
         };
-        uint32_t e[4][4];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-#pragma unroll
-            for (int f = 0; f < 4; ++f) {          // field f: d = f >> 1, s2 = f & 1
-                const uint32_t code = (grp[v] >> (6 * f)) & 63u;
-                e[v][f] = *(const uint32_t *)(lds + (code << es) + lane_off[v]);
-            }
-        }
 #pragma unroll
         for (int v = 0; v < 4; ++v)
 #pragma unroll
-            for (int f = 0; f < 4; ++f)
-                acc[v * 2 + (f >> 1)] = dot2<BF16>(e[v][f], (f & 1) ? xb : xa, acc[v * 2 + (f >> 1)]);
+            for (int f = 0; f < 4; ++f) {           // field f: d = f >> 1, s2 = f & 1
+                const uint32_t code = (grp[v] >> (6 * f)) & 63u;
+                e[v * 4 + f] = *(const uint32_t *)(lds + (code << es) + lane_off[v]);
+            }
     }
 }
 
+template <int B, bool BF16>
+__device__ __forceinline__ void quarter_dots(const uint32_t (&e)[16], uint32_t xa, uint32_t xb,
+                                             float (&acc)[8]) {
+    if constexpr (B == 4 || B == 3) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[v * 2 + (j >> 1)] = dot2<BF16>(e[v * 4 + j], (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
+    } else if constexpr (B == 2) {
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+            acc[a] = dot2<BF16>(e[a * 2], xa, acc[a]);
+            acc[a] = dot2<BF16>(e[a * 2 + 1], xb, acc[a]);
+        }
+    } else {
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {               // a = v * 2 + d: dwords (z, w) of entry v for d = 1
+            acc[a] = dot2<BF16>(e[a * 2], xa, acc[a]);
+            acc[a] = dot2<BF16>(e[a * 2 + 1], xb, acc[a]);
+        }
+    }
+}
+
+// A wavefront-uniform pointer pinned into scalar registers.  Loads written as
+// (uniform base + 32-bit lane offset) then keep that form; otherwise the loop
+// optimiser turns every such load into its own 64-bit per-lane pointer, carried in
+// vector registers across the K loop.
+typedef const __attribute__((address_space(1))) uint8_t *GlobalBytes;
+__device__ __forceinline__ GlobalBytes uniform_ptr(const uint8_t *ptr) {
+    const uint64_t b = (uint64_t)ptr;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    return (GlobalBytes)(((uint64_t)hi << 32) | lo);      // global, not generic: no flat loads
+}
+
 template <int B>
-__device__ __forceinline__ void load_quarter(uint32_t (&w)[B], const uint8_t *p) {
+__device__ __forceinline__ void load_quarter(uint32_t (&w)[B], GlobalBytes p) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    typedef const __attribute__((address_space(1))) u32x4 *G16;
+    typedef const __attribute__((address_space(1))) u32x2 *G8;
+    typedef const __attribute__((address_space(1))) uint32_t *G4;
     if constexpr (B == 4) {
-        const uint4 v = *(const uint4 *)p;
+        const u32x4 v = *(G16)p;
         w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
     } else if constexpr (B == 3) {
-        const uint32_t *q = (const uint32_t *)p;
+        G4 q = (G4)p;
         w[0] = q[0]; w[1] = q[1]; w[2] = q[2];
     } else if constexpr (B == 2) {
-        const uint2 v = *(const uint2 *)p;
+        const u32x2 v = *(G8)p;
         w[0] = v.x; w[1] = v.y;
     } else {
-        w[0] = *(const uint32_t *)p;
+        w[0] = *(G4)p;
     }
 }
 
@@ -416,7 +414,7 @@ struct LaneGeom {
 // Per-lane state of one stream pass between its phases.
 template <int B>
 struct StreamRegs {
-    static constexpr int kPrefetch = B == 4 ? 4 : (B == 3 ? 5 : 8);   // loads in flight per lane
+    static constexpr int kPrefetch = B == 4 ? 4 : 8;   // loads in flight per lane (a unit is 4*B bytes of it)
     static constexpr int kEDW = 1 << (TableShape<B>::kEntryLog2 - 2);
     uint32_t q[kPrefetch][B];
     uint32_t val[kEDW];      // this thread's table entry (fast path)
@@ -456,11 +454,18 @@ __device__ __forceinline__ void stream_issue(const GemvParams &p, const GemvSeg 
 #pragma unroll
         for (int s = 0; s < StreamRegs<B>::kEDW; ++s) r.val[s] = table_dword<B>(lut, item % E, s);
     }
+    // Every load is unconditional (a wavefront with fewer than PF units re-reads the
+    // first unit of the K range into the registers it will not consume), issued in
+    // the order of use and addressed as a uniform base plus one lane-constant
+    // offset: the compiler then knows how many loads are in flight at each point and
+    // waits for exactly the one a unit needs.
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int n = 0; n < PF; ++n) {
-#pragma unroll
-        for (int j = 0; j < B; ++j) r.q[n][j] = 0u;
-        if (n < r.my_units) load_quarter<B>(r.q[n], r.qrow + (r.lane0 + (uint32_t)n * r.step));
+        const uint8_t *base = n < r.my_units ? r.qrow + (size_t)n * r.step
+                                             : r.qrow - (size_t)gm.w * unit_bytes;
+        load_quarter<B>(r.q[n], uniform_ptr(base) + r.lane0);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -525,27 +530,62 @@ __device__ __forceinline__ void stream_loop(const GemvParams &p, const GemvSeg &
     }
     const uint32_t *xs32 = (const uint32_t *)(lds + p.lds_x);
     const int xi = gm.gsub * 32 + (gm.l & 3) * 8 + ((gm.l >> 2) & 3);   // + unit * gpi * 32
-    const bool perm = (es == 8);
-    for (int nb = 0; nb < r.my_units; nb += PF) {
+    auto lookups = [&](const uint32_t (&wq)[B], uint32_t (&e)[16]) {
+        quarter_lookups<B>(wq, lds, lane_off, es, e);
+    };
+    // The staged activations of consecutive units of this wavefront are xstep
+    // dwords apart; one running index serves every unit (a separate address per
+    // unrolled unit would be hoisted out of the loop and held in registers).
+    const int xstep = gm.nwaves * gm.gpi * 32;
+    int xo = gm.w * gm.gpi * 32 + xi;
+    auto dots = [&](const uint32_t (&e)[16]) {
+        quarter_dots<B, BF16>(e, xs32[xo], xs32[xo + 4], acc);
+        xo += xstep;
+        asm volatile("" : "+v"(xo));                          // keep it one running register
+    };
+    // The loop is cut so that every load inside its main part is unconditional; a
+    // conditional refill in a loop makes the compiler wait for all loads in flight
+    // at the loop head, which serialises the memory stream and the arithmetic.
+    const int U = r.my_units;
+    int nb = 0;
+    for (; nb + 2 * PF <= U; nb += PF) {                      // every refill exists
 #pragma unroll
         for (int n = 0; n < PF; ++n) {
-            const int m = nb + n;
-            if (m < r.my_units) {                   // uniform within the wavefront
-                uint32_t wq[B];
+            uint32_t e[16];
+            lookups(r.q[n], e);
+            __builtin_amdgcn_sched_barrier(0);                // refills stay where they are
+            load_quarter<B>(r.q[n], uniform_ptr(r.qrow + (size_t)(nb + n + PF) * r.step) + r.lane0);
+            __builtin_amdgcn_sched_barrier(0);
+            dots(e);
+        }
+    }
+    if (nb + PF >= U) {                                       // the last group, no refills
 #pragma unroll
-                for (int j = 0; j < B; ++j) wq[j] = r.q[n][j];
-                if (m + PF < r.my_units)
-                    load_quarter<B>(r.q[n], r.qrow + (r.lane0 + (uint32_t)(m + PF) * r.step));
-                const int xo = (gm.w + m * gm.nwaves) * gm.gpi * 32 + xi;
-                const uint32_t xa = xs32[xo];
-                const uint32_t xb = xs32[xo + 4];
-                if (B != 3 && perm)
-                    consume_quarter<B, BF16, (B != 3)>(wq, xa, xb, lds, lane_off, es, acc);
-                else
-                    consume_quarter<B, BF16, false>(wq, xa, xb, lds, lane_off, es, acc);
+        for (int n = 0; n < PF; ++n) {
+            if (nb + n < U) {                                 // uniform within the wavefront
+                uint32_t e[16];
+                lookups(r.q[n], e);
+                dots(e);
+            }
+        }
+    } else {
+        // A unit count that is not a multiple of PF: the rest runs with conditional
+        // refills (and the early waits they cause).
+        for (; nb < U; nb += PF) {
+#pragma unroll
+            for (int n = 0; n < PF; ++n) {
+                const int m = nb + n;
+                if (m < U) {
+                    uint32_t e[16];
+                    lookups(r.q[n], e);
+                    if (m + PF < U)
+                        load_quarter<B>(r.q[n], uniform_ptr(r.qrow + (size_t)(m + PF) * r.step) + r.lane0);
+                    dots(e);
+                }
             }
         }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0): nothing is in flight any more
 }
 
 // One stream pass whose loads were not issued ahead: all three phases in a row.
@@ -585,7 +625,7 @@ __device__ __forceinline__ int row_of(int cg, int a) {
 }
 
 template <bool BF16, int BFIX>
-__global__ void __launch_bounds__(kGemvMaxThreads, 4) gemv_kernel(const GemvParams p) {
+__global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
 
     // Read the weight descriptors straight from the kernel-argument segment
@@ -604,7 +644,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 4) gemv_kernel(const GemvPara
     LaneGeom gm;
     gm.tid = threadIdx.x;
     gm.nthreads = blockDim.x;
-    gm.w = gm.tid >> 6;
+    gm.w = __builtin_amdgcn_readfirstlane(gm.tid >> 6);
     gm.nwaves = gm.nthreads >> 6;
     gm.L = gm.tid & 63;
     const int lpg = 1 << p.lpg_log2;
@@ -624,53 +664,49 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 4) gemv_kernel(const GemvPara
 
     float *red = (float *)(lds + p.lds_red);        // [2][nwaves][32] row sums
     const int nout = p.silu_mul ? 2 : 1;
-    const float *staged_signs = nullptr, *staged_awq = nullptr;
-    const uint16_t *staged_x = nullptr;
-    bool staged = false;
-    // With one width for the whole launch, the very first pass issues its index
-    // and LUT loads BEFORE the activations are staged, so that the three kinds
-    // of loads travel together; later passes issue theirs when they start.
-    // Load order matters: activations, then LUT values, then index bytes, so that
-    // each consumer waits only for what was issued before it.
+    // With one width for the whole launch and a plain (unrotated) input, the first
+    // pass issues its loads in the order activations, LUT values, index bytes before
+    // anything is staged, so that the three kinds travel together and each consumer
+    // waits only for what was issued before it.  A rotated input is staged first: the
+    // rotation needs most of the register file, and index loads held across it would
+    // be spilled (and waited for) on the spot.
     constexpr int BF = BFIX != 0 ? BFIX : 4;
     constexpr int XV = 2;                           // 16-byte activation loads per thread
     StreamRegs<BF> first;
-    uint4 xv[XV];
     const uint16_t *x0 = sg.xsrc ? sg.xsrc : p.x;
     const bool x_ahead = BFIX != 0 && sg.signs == nullptr;      // uniform
     FLUTE_TRACE(0);
     if (x_ahead) {
+        uint4 xv[XV];
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
             const int j = (i * gm.nthreads + gm.tid) * 8;
-            xv[i] = make_uint4(0u, 0u, 0u, 0u);
-            if (j < kc) xv[i] = *(const uint4 *)(x0 + k0 + j);
+            xv[i] = *(const uint4 *)(x0 + k0 + (j < kc ? j : 0));
         }
+        if constexpr (BFIX != 0) stream_issue<BF>(p, sg, sg.st[0], gm, first);
+        FLUTE_TRACE(1);
+        uint16_t *xs = (uint16_t *)(lds + p.lds_x);
+#pragma unroll
+        for (int i = 0; i < XV; ++i) {
+            const int j = (i * gm.nthreads + gm.tid) * 8;
+            if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(xv[i], p.act_bf16);
+        }
+        for (int j = (XV * gm.nthreads + gm.tid) * 8; j < kc; j += gm.nthreads * 8)
+            *(uint4 *)(xs + j) = to_compute_type<BF16>(*(const uint4 *)(x0 + k0 + j), p.act_bf16);
+        // no barrier here: the one after the table build publishes both
+    } else {
+        stage_x<BF16>(p, x0, sg.signs, sg.awq, lds, k0, kc, gm.tid, gm.nthreads);
+        if constexpr (BFIX != 0) stream_issue<BF>(p, sg, sg.st[0], gm, first);
+        FLUTE_TRACE(1);
     }
-    if constexpr (BFIX != 0) stream_issue<BF>(p, sg, sg.st[0], gm, first);
-    FLUTE_TRACE(1);
+    const uint16_t *staged_x = x0;
+    const float *staged_signs = sg.signs, *staged_awq = sg.awq;
 
     for (int so = 0; so < nout; ++so) {
         const GemvSeg og = kp->seg[so == 1 ? 1 : si0];
         const uint16_t *xin = og.xsrc ? og.xsrc : p.x;
-        if (so == 0 && x_ahead) {
-            uint16_t *xs = (uint16_t *)(lds + p.lds_x);
-#pragma unroll
-            for (int i = 0; i < XV; ++i) {
-                const int j = (i * gm.nthreads + gm.tid) * 8;
-                if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(xv[i], p.act_bf16);
-            }
-            for (int j = (XV * gm.nthreads + gm.tid) * 8; j < kc; j += gm.nthreads * 8)
-                *(uint4 *)(xs + j) = to_compute_type<BF16>(*(const uint4 *)(x0 + k0 + j), p.act_bf16);
-            // no barrier here: the one after the table build publishes both
-            staged = true;
-            staged_x = xin;
-            staged_signs = og.signs;
-            staged_awq = og.awq;
-        } else if (!staged || xin != staged_x || og.signs != staged_signs ||
-                   og.awq != staged_awq) {
+        if (so > 0 && (xin != staged_x || og.signs != staged_signs || og.awq != staged_awq)) {
             stage_x<BF16>(p, xin, og.signs, og.awq, lds, k0, kc, gm.tid, gm.nthreads);
-            staged = true;
             staged_x = xin;
             staged_signs = og.signs;
             staged_awq = og.awq;
