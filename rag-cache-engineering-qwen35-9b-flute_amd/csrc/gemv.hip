@@ -160,7 +160,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
         if (per_cu < 1) per_cu = 1;
         const long fixed = kc * 2 + 4096;
         budget = 14;
-        for (int cand = 16; cand >= 14; --cand)
+        for (int cand = 15; cand >= 14; --cand)
             if (((1L << cand) + fixed) * per_cu <= kLdsPerCU) { budget = cand; break; }
     }
     for (int i = 0; i < count; ++i) {
@@ -218,7 +218,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
             gs.lut = (const uint16_t *)(st ? w.lut2 : w.lut1);
             gs.bits = st ? w.b2 : w.b1;
             int es = budget - entries_log2(gs.bits) - ngrp_log2;
-            if (es > 8) es = 8;
+            if (es > 7) es = 7;             // 32 replicas cover the 32 LDS banks
             if (es < entry_bytes_log2(gs.bits)) es = entry_bytes_log2(gs.bits);
             gs.es = es;
             const size_t tb = ((size_t)1 << (entries_log2(gs.bits) + es)) << ngrp_log2;
@@ -293,11 +293,11 @@ flute_status launch_typed(Plan &plan, hipStream_t stream) {
     return FLUTE_OK;
 }
 
-template <int LPGL, int NW, int ES, bool BF16, bool MULTI>
-flute_status launch_fast4m(Plan &plan, hipStream_t stream) {
+template <int LPGL, int NW, int PF, bool BF16>
+flute_status launch_fast4(Plan &plan, hipStream_t stream) {
     static bool attr_done = false;
     if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv4_kernel<LPGL, NW, ES, BF16, MULTI>,
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv4_kernel<LPGL, NW, PF, BF16>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
                                             (int)kLdsPerCU));
         attr_done = true;
@@ -309,25 +309,40 @@ flute_status launch_fast4m(Plan &plan, hipStream_t stream) {
     }
 #endif
     dim3 grid(plan.grid_x, plan.p.split);
-    hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, ES, BF16, MULTI>), grid, dim3(NW * 64),
-                       plan.lds_bytes, stream, plan.p);
+    hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, PF, BF16>), grid, dim3(NW * 64), plan.lds_bytes,
+                       stream, plan.p);
     FLUTE_HIP_CHECK(hipGetLastError());
     return FLUTE_OK;
 }
 
-template <int LPGL, int NW, int ES, bool BF16>
-flute_status launch_fast4(Plan &plan, hipStream_t stream) {
-    const bool multi = plan.p.nsegs > 1 && !plan.p.silu_mul;
-    return multi ? launch_fast4m<LPGL, NW, ES, BF16, true>(plan, stream)
-                 : launch_fast4m<LPGL, NW, ES, BF16, false>(plan, stream);
+// Loads a lane keeps in flight: the largest of 4, 3, 2 that divides the units of a
+// wavefront (no partial group in the K loop); 4 when the wavefronts differ or
+// nothing divides (that case runs the kernel's conservative tail).
+int pick_prefetch(const Plan &plan, int nw) {
+    const int gpi = 64 >> plan.p.lpg_log2;
+    const int units = plan.p.gs_tiles / gpi;
+    int pf = env_int("FLUTE_GEMV4_PF", 0);
+    if (pf >= 2 && pf <= 4) return pf;
+    if (units % nw) return 4;
+    const int u = units / nw;
+    for (int cand : {4, 3, 2})
+        if (u % cand == 0 || u < cand) return cand;
+    return 4;
+}
+
+template <int LPGL, int NW, bool BF16>
+flute_status launch_fast4_pf(Plan &plan, hipStream_t stream) {
+    switch (pick_prefetch(plan, NW)) {
+        case 2: return launch_fast4<LPGL, NW, 2, BF16>(plan, stream);
+        case 3: return launch_fast4<LPGL, NW, 3, BF16>(plan, stream);
+        default: return launch_fast4<LPGL, NW, 4, BF16>(plan, stream);
+    }
 }
 
 template <int LPGL, bool BF16>
-flute_status launch_fast4_shape(Plan &plan, int nw, int es, hipStream_t stream) {
-    if (nw == 4) return es == 8 ? launch_fast4<LPGL, 4, 8, BF16>(plan, stream)
-                                : launch_fast4<LPGL, 4, 7, BF16>(plan, stream);
-    return es == 8 ? launch_fast4<LPGL, 8, 8, BF16>(plan, stream)
-                   : launch_fast4<LPGL, 8, 7, BF16>(plan, stream);
+flute_status launch_fast4_shape(Plan &plan, int nw, hipStream_t stream) {
+    return nw == 4 ? launch_fast4_pf<LPGL, 4, BF16>(plan, stream)
+                   : launch_fast4_pf<LPGL, 8, BF16>(plan, stream);
 }
 
 template <bool BF16>
@@ -344,12 +359,12 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         }
     }
     const int nw = plan.threads / 64;
-    if (bits == 4 && one_group && (es == 7 || es == 8) && (nw == 4 || nw == 8) &&
+    if (bits == 4 && one_group && es == 7 && (nw == 4 || nw == 8) &&
         env_int("FLUTE_GEMV_NO_FAST", 0) == 0) {
         switch (plan.p.lpg_log2) {
-            case 4: return launch_fast4_shape<4, BF16>(plan, nw, es, stream);
-            case 5: return launch_fast4_shape<5, BF16>(plan, nw, es, stream);
-            default: return launch_fast4_shape<6, BF16>(plan, nw, es, stream);
+            case 4: return launch_fast4_shape<4, BF16>(plan, nw, stream);
+            case 5: return launch_fast4_shape<5, BF16>(plan, nw, stream);
+            default: return launch_fast4_shape<6, BF16>(plan, nw, stream);
         }
     }
     switch (bits) {

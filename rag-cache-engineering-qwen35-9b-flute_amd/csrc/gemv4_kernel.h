@@ -12,26 +12,26 @@ namespace flute {
 
 // LPGL = log2(lanes per 64-k tile) = log2(2 * rows per workgroup): 4, 5, 6.
 // NW   = wavefronts per workgroup.
-// ES   = log2(table stride): 8 (v_perm addressing, 64 KB) or 7 (32 KB).
-// MULTI = several independent weights share the launch (the descriptor is then
-//         picked by grid column, which costs a dependent scalar load).
-template <int LPGL, int NW, int ES, bool BF16, bool MULTI>
-// Three wavefronts per SIMD (168 registers), except where the 64 KB table already
-// limits a CU to two four-wavefront workgroups.
-__global__ void __launch_bounds__(NW * 64, (NW == 4 && ES == 8) ? 2 : 3)
-    gemv4_kernel(const GemvParams p) {
+// PF   = index loads a lane keeps in flight (2, 3 or 4).  A few loads per
+//        wavefront, refilled as they are consumed, serve every wavefront of the grid
+//        in turn; a deep queue (a wavefront's whole K range requested at once) is
+//        served wavefront by wavefront, and the last ones served start their
+//        arithmetic when the memory stream is already over.  The host picks the
+//        largest PF that divides the units of a wavefront, so that the K loop has no
+//        partial group.
+// The table stride is 128 bytes (32 replicas of a 4-byte entry, 32 KB): three
+// four-wavefront workgroups fit a CU.
+template <int LPGL, int NW, int PF, bool BF16>
+__global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
+    constexpr int ES = 7;
     constexpr int NT = NW * 64;
     constexpr int LPG = 1 << LPGL;
     constexpr int GPI = 64 >> LPGL;                 // 64-k tiles per wavefront load
     constexpr int RW = LPG >> 1;                    // rows per workgroup
     constexpr int SPT = 128 / RW;                   // row slices per tile
-    constexpr int PF = NW == 4 ? 8 : 4;             // wavefront loads in flight per lane
     constexpr int XV = 2;                           // 16-byte activation loads per thread
-#ifndef FLUTE_GEMV4_PF0
-#define FLUTE_GEMV4_PF0 2
-#endif
-    constexpr int PF0 = FLUTE_GEMV4_PF0 < PF ? FLUTE_GEMV4_PF0 : PF;   // index loads ahead of the table
+    constexpr int PF0 = 1;                          // index loads issued ahead of the table build
     constexpr int STRIDE = 1 << ES;                 // table bytes per entry
     constexpr int CHUNKS = STRIDE / 16;             // 16-byte pieces of one entry's replicas
     constexpr int SHARES = NT / 256;                // threads per table entry
@@ -40,8 +40,9 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && ES == 8) ? 2 : 3)
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     warm_kernargs<(int)sizeof(GemvParams)>(kp);
+    // several independent weights in one launch: the descriptor is picked by grid column
     int si0 = 0;
-    if (MULTI && !p.silu_mul) {
+    if (p.nsegs > 1 && !p.silu_mul) {
 #pragma unroll
         for (int i = 1; i < kGemvMaxSegs; ++i)
             if (i < p.nsegs && (int)blockIdx.x >= p.seg[i].col0) si0 = i;
@@ -77,7 +78,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && ES == 8) ? 2 : 3)
     // instead of being added after every v_perm.
     typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-    const uint32_t slot = lds_base + (ES == 8 ? (uint32_t)L * 4u : (uint32_t)(L & 31) * 4u);
+    const uint32_t slot = lds_base + (uint32_t)(L & 31) * 4u;
     const int e_own = tid & 255;                    // table entry this thread writes
     const int share = tid >> 8;
 
@@ -260,13 +261,7 @@ __global__ void __launch_bounds__(NW * 64, (NW == 4 && ES == 8) ? 2 : 3)
                 const uint32_t wv = v == 0 ? qv.x : v == 1 ? qv.y : v == 2 ? qv.z : qv.w;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {       // byte j: d = j >> 1, s2 = j & 1
-                    uint32_t addr;
-                    if constexpr (ES == 8) {
-                        addr = __builtin_amdgcn_perm(wv, slot, 0x03020000u | ((4u + j) << 8));
-                    } else {
-                        addr = (((wv >> (8 * j)) & 0xffu) << ES) + slot;
-                    }
-                    e[v][j] = *(LdsWord)addr;
+                    e[v][j] = *(LdsWord)((((wv >> (8 * j)) & 0xffu) << ES) + slot);
                 }
             }
         };
