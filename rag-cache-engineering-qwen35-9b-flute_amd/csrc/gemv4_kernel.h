@@ -129,6 +129,12 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     };
 
     FLUTE_TRACE(0);
+    // Wavefront priority falls as a workgroup advances: 3 in the prologue, 2 while
+    // there is more to stream, 1 in the last group, 0 from the fold on.  A SIMD holds
+    // one wavefront of each resident workgroup and serves the oldest first; without
+    // this the workgroup that arrived last on a CU lags through the whole launch and
+    // ends more than a microsecond after the first.
+    __builtin_amdgcn_s_setprio(3);
     // ---- first pass: activations, LUT values and the first index bytes.  The order
     //      of the loads is the order they are needed in, and the scheduler is kept
     //      from changing it: a wait for an early load also waits for everything
@@ -277,6 +283,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                         dot2<BF16>(e[v][j], (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
         };
         int nb = 0;
+        __builtin_amdgcn_s_setprio(2);
         for (; nb + 2 * PF <= my_units; nb += PF) {          // every refill exists
 #pragma unroll
             for (int n = 0; n < PF; ++n) {
@@ -290,6 +297,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 dots(e, nb + n);
             }
         }
+        if (!has_next) __builtin_amdgcn_s_setprio(1);
         if (nb + PF == my_units && has_next) {                // a full last group, refilled
 #pragma unroll                                                //   from the next pass
             for (int n = 0; n < PF; ++n) {
@@ -331,6 +339,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         if (!has_next) FLUTE_TRACE(3); else if (first) FLUTE_TRACE(6);
 #endif
 
+        if (!has_next) __builtin_amdgcn_s_setprio(0);
         // ---- end of an output: fold the lanes that share rows ------------------------
         if (nso != so) {
 #pragma unroll

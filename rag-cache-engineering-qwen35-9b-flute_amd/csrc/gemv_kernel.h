@@ -548,6 +548,7 @@ __device__ __forceinline__ void stream_loop(const GemvParams &p, const GemvSeg &
     // at the loop head, which serialises the memory stream and the arithmetic.
     const int U = r.my_units;
     int nb = 0;
+    __builtin_amdgcn_s_setprio(2);
     for (; nb + 2 * PF <= U; nb += PF) {                      // every refill exists
 #pragma unroll
         for (int n = 0; n < PF; ++n) {
@@ -633,6 +634,10 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     // offset instead of a select chain over every field of every descriptor.
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     warm_kernargs<(int)sizeof(GemvParams)>(kp);
+    // Wavefront priority falls as a workgroup advances (3 in the prologue, 2 in the
+    // K loops, 0 from the last fold on): a SIMD serves its oldest wavefront first, and
+    // the workgroup that arrived last on a CU would otherwise lag through the launch.
+    __builtin_amdgcn_s_setprio(3);
     int si0 = 0;
     if (!p.silu_mul) {
 #pragma unroll
@@ -745,6 +750,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
                 red[(so * gm.nwaves + gm.w) * 32 + (gm.L >> 4) * 8 + a] = acc[a];
         }
     }
+    __builtin_amdgcn_s_setprio(0);
     __syncthreads();
 
     // ---- one thread per owned row: fold the wavefronts in fixed order ----------
