@@ -181,37 +181,51 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             q[n] = unit_load(qrow, n);
             __builtin_amdgcn_sched_barrier(0);
         }
-    } else {
-        // A long K range, or a rotated input: everything the table and the staged
-        // activations need is fetched and written first (the index registers carry the
-        // activations meanwhile), then the index loads start.
-        if (x_direct) {
+    } else if (x_direct) {
+        // A long K range: everything the table and the staged activations need is
+        // fetched and written first (the index registers carry the activations
+        // meanwhile), then the index loads start.
 #pragma unroll
-            for (int n = 0; n < PF; ++n) {
-                const int j = (n * NT + tid) * 8;
-                q[n] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
-            }
+        for (int n = 0; n < PF; ++n) {
+            const int j = (n * NT + tid) * 8;
+            q[n] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
         }
         __builtin_amdgcn_sched_barrier(0);
         lo = lut[e_own & 15];
         hi = lut[e_own >> 4];
         __builtin_amdgcn_sched_barrier(0);
         FLUTE_TRACE(1);
-        if (x_direct) {
 #pragma unroll
-            for (int n = 0; n < PF; ++n) {
-                const int j = (n * NT + tid) * 8;
-                if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(q[n], p.act_bf16);
-            }
-            for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8)
-                *(uint4 *)(xs + j) =
-                    to_compute_type<BF16>(*(const uint4 *)(staged_x + k0 + j), p.act_bf16);
-        } else {
-            stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
+        for (int n = 0; n < PF; ++n) {
+            const int j = (n * NT + tid) * 8;
+            if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(q[n], p.act_bf16);
         }
+        for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8)
+            *(uint4 *)(xs + j) =
+                to_compute_type<BF16>(*(const uint4 *)(staged_x + k0 + j), p.act_bf16);
         write_table(lo, hi);
         __builtin_amdgcn_sched_barrier(0);
         first_units(qrow, q);
+    } else {
+        // A rotated input: the LUT values and the first index loads travel while the
+        // rotation runs.
+        lo = lut[e_own & 15];
+        hi = lut[e_own >> 4];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int n = 0; n < PF0; ++n) {
+            q[n] = unit_load(qrow, n);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        FLUTE_TRACE(1);
+        stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
+        write_table(lo, hi);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int n = PF0; n < PF; ++n) {
+            q[n] = unit_load(qrow, n);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 
     float acc[8];

@@ -342,6 +342,98 @@ __device__ __forceinline__ void rotated_in8(float *buf, int j, const uint16_t *x
     for (int q = 0; q < 8; ++q) buf[s0 ^ q] = f[q];
 }
 
+// Equal rotation blocks of at most 256 columns, without the fp32 LDS buffer: a thread
+// holds eight consecutive columns, so the stages of length 1, 2, 4 are butterflies
+// between its own registers, and the stages of length 8 .. block/2 pair it with the
+// lane whose number differs in one bit (ds_swizzle, the LDS crossbar without a memory
+// access).  The lower lane of a pair keeps a + b and the upper a - b, formed as
+// fma(mine, +-1, other): the product is exact, so every value sees the same single
+// rounding per stage, in the same ascending order, as in the buffered butterfly and
+// the result is bit-identical.  The loads of all (at most two) steps of a thread go
+// out before the first butterfly: one memory round trip for the whole rotation, no
+// barrier.  Lanes of one block are in the same step, so a step's partners are active.
+template <bool BF16>
+__device__ __forceinline__ void rotate_blocks_inwave(const uint16_t *x, const float *signs,
+                                                     const float *awq, uint16_t *xs, int k0,
+                                                     int kc, int block, int act_bf16, int tid,
+                                                     int nthreads) {
+    const int nst = 31 - __builtin_clz((unsigned)block);
+    const float inv = inv_sqrt_pow2(nst);
+    const int lane = tid & 63;
+    const int pair_lanes = block >> 3;                 // lanes of one block: 4 .. 32
+    for (int j0 = tid * 8; j0 < kc; j0 += 2 * nthreads * 8) {
+        float f[2][8], sg[2][8], sc[2][8];
+        const int j1 = j0 + nthreads * 8;
+        const bool two = j1 < kc;                      // same for every lane of a block
+        load_act8(x, k0 + j0, act_bf16, f[0]);
+        load_act8(x, k0 + (two ? j1 : j0), act_bf16, f[1]);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            sg[0][q] = signs[k0 + j0 + q];
+            sg[1][q] = signs[k0 + (two ? j1 : j0) + q];
+        }
+        if (awq) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                sc[0][q] = awq[k0 + j0 + q];
+                sc[1][q] = awq[k0 + (two ? j1 : j0) + q];
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                f[0][q] *= sc[0][q];
+                f[1][q] *= sc[1][q];
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int len = 1; len < 8; len <<= 1) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    if ((q & len) == 0) {
+                        const float a = f[h][q], c = f[h][q | len];
+                        f[h][q] = a + c;
+                        f[h][q | len] = a - c;
+                    }
+                }
+            }
+        }
+        // and_mask 0x1f, or_mask 0, xor_mask m: lane ^ m inside each half of the wavefront
+#define FLUTE_XOR_STAGE(m)                                                                   \
+        if (pair_lanes > (m)) {                                                              \
+            const float sgn = (lane & (m)) ? -1.0f : 1.0f;                                   \
+            _Pragma("unroll") for (int h = 0; h < 2; ++h)                                    \
+                _Pragma("unroll") for (int q = 0; q < 8; ++q) {                              \
+                    const float other = __int_as_float(__builtin_amdgcn_ds_swizzle(          \
+                        __float_as_int(f[h][q]), ((m) << 10) | 0x1f));                       \
+                    f[h][q] = fmaf(f[h][q], sgn, other);                                     \
+                }                                                                            \
+        }
+        FLUTE_XOR_STAGE(1)
+        FLUTE_XOR_STAGE(2)
+        FLUTE_XOR_STAGE(4)
+        FLUTE_XOR_STAGE(8)
+        FLUTE_XOR_STAGE(16)
+#undef FLUTE_XOR_STAGE
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (h == 1 && !two) break;
+            uint32_t o[4];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                float t = f[h][q] * sg[h][q] * inv;
+                if (awq) t = t / sc[h][q];
+                const uint16_t a = round_act(t, act_bf16);
+                const float back = act_bf16 ? bf2f(a) : h2f(a);
+                const uint32_t v = BF16 ? f2bf(back) : f2h(back);
+                if (q & 1) o[q >> 1] |= v << 16;
+                else o[q >> 1] = v;
+            }
+            *(uint4 *)(xs + (h ? j1 : j0)) = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+    }
+}
+
 // Stage the activation slice [k0, k0 + kc) into LDS as 16-bit values of the
 // compute type (the LUT's type), 16 bytes per thread per step so that the whole
 // slice is one round trip to memory.  With signs, the rotation of every segment
@@ -360,6 +452,11 @@ __device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *sig
         return;
     }
     float *buf = (float *)lds;
+    if (p.fht_block > 0 && p.fht_block <= 256) {
+        rotate_blocks_inwave<BF16>(x, signs, awq, xs, k0, kc, p.fht_block, p.act_bf16, tid, nthreads);
+        __syncthreads();
+        return;
+    }
     if (p.fht_block > 0) {
         // equal blocks: the slice is a whole number of blocks
 #pragma unroll 2
