@@ -269,6 +269,21 @@ __device__ __forceinline__ void load_quarter(uint32_t (&w)[B], GlobalBytes p) {
     }
 }
 
+// Eight consecutive floats (signs, scales), as two 16-byte loads when the array is
+// 16-byte aligned (k is a multiple of 8).  Element-wise loads here each touch 64
+// lanes x 4 bytes spread over 2 KB, and the vector memory pipe is then the bottleneck
+// of the whole rotation.
+__device__ __forceinline__ void load_f8(const float *src, int k, float (&v)[8]) {
+    if (((uintptr_t)src & 15) == 0) {                  // uniform
+        const float4 a = *(const float4 *)(src + k), b = *(const float4 *)(src + k + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[q] = src[k + q];
+    }
+}
+
 // Eight consecutive activations (16 bytes) as floats.
 __device__ __forceinline__ void load_act8(const uint16_t *x, int k, int is_bf16, float (&f)[8]) {
     const uint4 v = *(const uint4 *)(x + k);
@@ -304,12 +319,8 @@ __device__ __forceinline__ void rotated_out8(const float *buf, int j, const floa
                                              const float *awq, int g, float inv, int act_bf16,
                                              uint16_t *dst) {
     float sg[8], sc[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) sg[q] = signs[g + q];
-    if (awq) {
-#pragma unroll
-        for (int q = 0; q < 8; ++q) sc[q] = awq[g + q];
-    }
+    load_f8(signs, g, sg);
+    if (awq) load_f8(awq, g, sc);
     uint32_t o[4];
     const int s0 = fht_slot(j);                        // j is a multiple of 8: slot(j + q) = s0 ^ q
 #pragma unroll
@@ -332,8 +343,7 @@ __device__ __forceinline__ void rotated_in8(float *buf, int j, const uint16_t *x
     float f[8], sc[8];
     load_act8(x, g, act_bf16, f);
     if (awq) {
-#pragma unroll
-        for (int q = 0; q < 8; ++q) sc[q] = awq[g + q];
+        load_f8(awq, g, sc);
 #pragma unroll
         for (int q = 0; q < 8; ++q) f[q] *= sc[q];
     }
@@ -367,17 +377,11 @@ __device__ __forceinline__ void rotate_blocks_inwave(const uint16_t *x, const fl
         const bool two = j1 < kc;                      // same for every lane of a block
         load_act8(x, k0 + j0, act_bf16, f[0]);
         load_act8(x, k0 + (two ? j1 : j0), act_bf16, f[1]);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            sg[0][q] = signs[k0 + j0 + q];
-            sg[1][q] = signs[k0 + (two ? j1 : j0) + q];
-        }
+        load_f8(signs, k0 + j0, sg[0]);
+        load_f8(signs, k0 + (two ? j1 : j0), sg[1]);
         if (awq) {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                sc[0][q] = awq[k0 + j0 + q];
-                sc[1][q] = awq[k0 + (two ? j1 : j0) + q];
-            }
+            load_f8(awq, k0 + j0, sc[0]);
+            load_f8(awq, k0 + (two ? j1 : j0), sc[1]);
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 f[0][q] *= sc[0][q];
@@ -434,6 +438,129 @@ __device__ __forceinline__ void rotate_blocks_inwave(const uint16_t *x, const fl
     }
 }
 
+// One rotation segment of b = 512 .. 16 * nthreads columns starting at column `off`,
+// all of it inside the staged slice.  The first nine stages (lengths 1 .. 256) run as
+// in rotate_blocks_inwave, the last of them against the lane 32 away; what is left
+// (lengths 512 .. b/2, at most four stages) is one pass over the fp32 buffer in LDS.
+// Same butterflies in the same ascending order as fht_lds alone: bit-identical.
+// Against the buffered transform this halves the LDS traffic, drops two of five
+// barriers and needs one memory round trip instead of three.
+template <bool BF16>
+__device__ __forceinline__ void rotate_segment_fast(const uint16_t *x, const float *signs,
+                                                    const float *awq, float *buf, uint16_t *xs,
+                                                    int off, int xs_off, int b, int act_bf16,
+                                                    int tid, int nthreads) {
+    const int nst = 31 - __builtin_clz((unsigned)b);
+    const float inv = inv_sqrt_pow2(nst);
+    const int lane = tid & 63;
+    const int j0 = tid * 8, j1 = j0 + nthreads * 8;
+    const bool one = j0 < b, two = j1 < b;             // whole wavefronts: b/8 is a multiple of 64
+    float f[2][8], sg[2][8], sc[2][8];
+    if (one) {
+        load_act8(x, off + j0, act_bf16, f[0]);
+        load_act8(x, off + (two ? j1 : j0), act_bf16, f[1]);
+        load_f8(signs, off + j0, sg[0]);
+        load_f8(signs, off + (two ? j1 : j0), sg[1]);
+        if (awq) {
+            load_f8(awq, off + j0, sc[0]);
+            load_f8(awq, off + (two ? j1 : j0), sc[1]);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                f[0][q] *= sc[0][q];
+                f[1][q] *= sc[1][q];
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int len = 1; len < 8; len <<= 1) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    if ((q & len) == 0) {
+                        const float a = f[h][q], c = f[h][q | len];
+                        f[h][q] = a + c;
+                        f[h][q | len] = a - c;
+                    }
+                }
+            }
+        }
+#define FLUTE_XOR_STAGE(m)                                                                   \
+        {                                                                                    \
+            const float sgn = (lane & (m)) ? -1.0f : 1.0f;                                   \
+            _Pragma("unroll") for (int h = 0; h < 2; ++h)                                    \
+                _Pragma("unroll") for (int q = 0; q < 8; ++q) {                              \
+                    const float other = __int_as_float(__builtin_amdgcn_ds_swizzle(          \
+                        __float_as_int(f[h][q]), ((m) << 10) | 0x1f));                       \
+                    f[h][q] = fmaf(f[h][q], sgn, other);                                     \
+                }                                                                            \
+        }
+        FLUTE_XOR_STAGE(1)
+        FLUTE_XOR_STAGE(2)
+        FLUTE_XOR_STAGE(4)
+        FLUTE_XOR_STAGE(8)
+        FLUTE_XOR_STAGE(16)
+#undef FLUTE_XOR_STAGE
+        {
+            const float sgn = (lane & 32) ? -1.0f : 1.0f;
+            const int partner = (lane ^ 32) << 2;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const float other = __int_as_float(
+                        __builtin_amdgcn_ds_bpermute(partner, __float_as_int(f[h][q])));
+                    f[h][q] = fmaf(f[h][q], sgn, other);
+                }
+        }
+    }
+    if (nst > 9) {                                     // uniform: stages of length 512 and up
+        if (one) {
+            const int s0 = fht_slot(j0), s1 = fht_slot(j1);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) buf[s0 ^ q] = f[0][q];
+            if (two) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) buf[s1 ^ q] = f[1][q];
+            }
+        }
+        __syncthreads();
+        switch (nst - 9) {
+            case 1: fht_pass<1>(buf, b, 9, tid, nthreads); break;
+            case 2: fht_pass<2>(buf, b, 9, tid, nthreads); break;
+            case 3: fht_pass<3>(buf, b, 9, tid, nthreads); break;
+            default: fht_pass<4>(buf, b, 9, tid, nthreads); break;
+        }
+        __syncthreads();
+        if (one) {
+            const int s0 = fht_slot(j0), s1 = fht_slot(j1);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) f[0][q] = buf[s0 ^ q];
+            if (two) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) f[1][q] = buf[s1 ^ q];
+            }
+        }
+    }
+    if (one) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (h == 1 && !two) break;
+            uint32_t o[4];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                float t = f[h][q] * sg[h][q] * inv;
+                if (awq) t = t / sc[h][q];
+                const uint16_t a = round_act(t, act_bf16);
+                const float back = act_bf16 ? bf2f(a) : h2f(a);
+                const uint32_t v = BF16 ? f2bf(back) : f2h(back);
+                if (q & 1) o[q >> 1] |= v << 16;
+                else o[q >> 1] = v;
+            }
+            *(uint4 *)(xs + xs_off + (h ? j1 : j0)) = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+    }
+}
+
 // Stage the activation slice [k0, k0 + kc) into LDS as 16-bit values of the
 // compute type (the LUT's type), 16 bytes per thread per step so that the whole
 // slice is one round trip to memory.  With signs, the rotation of every segment
@@ -477,7 +604,12 @@ __device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *sig
         const int nst = 31 - __builtin_clz((unsigned)rem);
         const int b = 1 << nst;
         const int lo = max(off, k0), hi = min(off + b, k0 + kc);
-        if (lo < hi) {                             // uniform across the workgroup
+        if (lo < hi && lo == off && hi == off + b && b >= 512 && b <= 16 * nthreads &&
+            (nthreads & 63) == 0 && nst <= 13) {
+            rotate_segment_fast<BF16>(x, signs, awq, buf, xs, off, off - k0, b, p.act_bf16, tid,
+                                      nthreads);
+            __syncthreads();                       // scratch is reused by the next segment
+        } else if (lo < hi) {                      // uniform across the workgroup
 #pragma unroll 2
             for (int j = tid * 8; j < b; j += nthreads * 8)
                 rotated_in8(buf, j, x, off + j, awq, p.act_bf16);
