@@ -48,16 +48,21 @@ struct Plan {
 // the split stays 1 as long as the row slices alone give every CU at least two
 // workgroups.
 void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *waves) {
+    bool exact_tiling = false;
     int best_rw = env_int("FLUTE_GEMV_RW", 0);
     if (best_rw != 8 && best_rw != 16 && best_rw != 32) {
         best_rw = 8;
         for (int cand : {32, 16, 8}) {
             if (rows / cand >= 2 * kNumCU + kNumCU / 2) { best_rw = cand; break; }
         }
-        // A grid of exactly one, two or three 16-row workgroups per CU measured best
-        // where it exists (4096 rows: 256 eight-wavefront workgroups, 8.5 us against
-        // 9.2 us for 512 eight-row ones at K = 12288).
-        if (rows % (16 * kNumCU) == 0 && rows / (16 * kNumCU) <= 3) best_rw = 16;
+        // A grid of exactly one or two 16-row workgroups per CU, unsplit, measured best
+        // where K is long enough to give each of them eight wavefronts (4096 rows at
+        // K = 12288: 256 workgroups, 8.5 us against 9.2 us for 512 eight-row ones and
+        // 9.5 us for 768 with a three-way K split).
+        if (rows % (16 * kNumCU) == 0 && rows / (16 * kNumCU) <= 2 && G / 2 >= 64) {
+            best_rw = 16;
+            exact_tiling = true;
+        }
     }
     int sp = split_req;
     if (sp > 0) {
@@ -68,7 +73,7 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
         sp = 1;
         const long slices = rows / best_rw;
         const int gpi = 32 / best_rw;
-        if (slices < 2 * kNumCU) {
+        if (slices < 2 * kNumCU && !exact_tiling) {
             // narrow output: split K until the grid reaches about three workgroups per CU
             long best_cost = -1;
             for (int d = 1; d <= G; ++d) {
