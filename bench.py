@@ -33,7 +33,7 @@ H, I, GS = 4096, 12288, 128
 # HBM bytes one launch of the merged gate+up kernel moves, from FETCH_SIZE and WRITE_SIZE
 # counter runs of this file scaled by a copy of known size (--calibrate-copy); the readings
 # are kept in profiles/gemv4_gate_up_hbm_traffic.txt.  Only valid for the default workload.
-TRAFFIC_GATE_UP_BYTES = 50857700
+TRAFFIC_GATE_UP_BYTES = 50790600
 
 
 def _weights(torch, N, K, gen, dev, lut_dtype):

@@ -368,7 +368,12 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         }
     }
     const int nw = plan.threads / 64;
-    if (bits == 4 && one_group && es == 7 && (nw == 4 || nw == 8) &&
+    // the lean kernel stages the activations once: gate and up must share input and rotation
+    const bool one_input = !plan.p.silu_mul ||
+                           (plan.p.seg[0].xsrc == plan.p.seg[1].xsrc &&
+                            plan.p.seg[0].signs == plan.p.seg[1].signs &&
+                            plan.p.seg[0].awq == plan.p.seg[1].awq);
+    if (bits == 4 && one_group && one_input && es == 7 && (nw == 4 || nw == 8) &&
         env_int("FLUTE_GEMV_NO_FAST", 0) == 0) {
         switch (plan.p.lpg_log2) {
             case 4: return launch_fast4_shape<4, BF16>(plan, nw, stream);
