@@ -175,3 +175,36 @@ def test_block_rotation_mode():
     y = _run(w, x, signs=signs, rot_block=128).cpu()
     xo = O.block_fht_reference(x, 128, signs)
     assert rel_l2(y, _exact(w, xo).half()) <= TOL
+
+
+# Unit counts per wavefront that are and are not a multiple of the prefetch depth, K ranges
+# shorter than one load per wavefront, and K ranges beyond the activation registers of the
+# prologue: every variant of the K loop (main part, last group, conservative tail) and both
+# activation staging paths.
+@pytest.mark.parametrize("K", [64, 128, 192, 320, 448, 832, 1792, 2560, 5120, 6144, 8192, 16384])
+@pytest.mark.parametrize("N,bits,bits2", [(256, 4, 0), (2048, 4, 0), (512, 4, 4), (512, 2, 0)])
+def test_k_sweep_covers_every_loop_variant(K, N, bits, bits2):
+    if N == 2048 and K > 8192:
+        pytest.skip("covered by the narrower rows")
+    w = make_weight(N, K, bits, 128, seed=K + N + bits, bits2=bits2, device=DEV)
+    x = make_x(1, K, seed=11)
+    y = _run(w, x).cpu()
+    assert rel_l2(y, _exact(w, x).half()) <= TOL
+    assert torch.equal(y, _run(w, x).cpu())
+
+
+@pytest.mark.parametrize("block", [32, 64, 128, 256, 512, 1024])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_block_rotation_is_bit_identical_to_rotate_then_gemv(block, dtype):
+    """Blocks up to 256 columns run in registers and lane swizzles, larger ones in the LDS
+    buffer; both must produce the bits of the standalone rotation kernel."""
+    from flute_extended import _C
+    N, K = 512, 4096
+    w = make_weight(N, K, 4, 128, seed=block, act_dtype=dtype, device=DEV)
+    x = make_x(1, K, seed=12, dtype=dtype)
+    signs = O.rotation_signs(K, block)
+    fused = _run(w, x, signs=signs, rot_block=block)
+    xr = _C.fht_forward(x.to(DEV), signs.to(DEV), block)
+    assert torch.equal(fused, _run(w, xr.cpu()))
+    xo = O.block_fht_reference(x, block, signs)
+    assert rel_l2(fused.cpu(), _exact(w, xo).to(dtype)) <= (TOL if dtype == torch.float16 else 4e-3)
