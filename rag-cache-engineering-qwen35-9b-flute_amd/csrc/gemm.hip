@@ -219,7 +219,8 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
         const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
         hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
                            (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
-                           (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16));
+                           (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
+                           (int)((((uintptr_t)A & 3) == 0) && (lda % 2 == 0)));
         FLUTE_HIP_CHECK(hipGetLastError());
     }
     if (w->R > 0) {

@@ -67,7 +67,7 @@ struct GemmParams {
 // Activation pre-pass: Ap[g][j][mb][lane][slot] in the LUT's 16-bit type.
 __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t *Ap, int M,
                                                         int64_t lda, int G, int mblk,
-                                                        int in_bf16, int out_bf16) {
+                                                        int in_bf16, int out_bf16, int pairs) {
     const int64_t total = (int64_t)G * 2 * mblk * 64;
     for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total;
          o += (int64_t)gridDim.x * blockDim.x) {
@@ -82,7 +82,16 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t 
 #pragma unroll
             for (int s = 0; s < 4; ++s) {              // s = ktl*2 + s2
                 const int k = g * 64 + (2 * j + (s >> 1)) * 16 + 2 * kg + 8 * (s & 1);
-                uint16_t a0 = A[m * lda + k], a1 = A[m * lda + k + 1];
+                // k is even: one 32-bit load per pair where the rows are 4-byte aligned
+                uint16_t a0, a1;
+                if (pairs) {
+                    const uint32_t pair = *(const uint32_t *)(A + m * lda + k);
+                    a0 = (uint16_t)(pair & 0xffffu);
+                    a1 = (uint16_t)(pair >> 16);
+                } else {
+                    a0 = A[m * lda + k];
+                    a1 = A[m * lda + k + 1];
+                }
                 if (in_bf16 != out_bf16) {
                     a0 = round_act(in_bf16 ? bf2f(a0) : h2f(a0), out_bf16);
                     a1 = round_act(in_bf16 ? bf2f(a1) : h2f(a1), out_bf16);
