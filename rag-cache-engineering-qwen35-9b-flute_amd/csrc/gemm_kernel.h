@@ -269,7 +269,10 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     const int64_t jstep = (int64_t)p.mblk_pad * 64;    // u4 units between the halves of a tile
     // Ap is padded to whole workgroups of blocks (zeros), so every block index below
     // gridDim.y * MW * MB is loadable.
-    const u4_t *ap = p.Ap + ((int64_t)g0 * 2 * p.mblk_pad + mb0) * 64 + lane;
+    // A wavefront without tiles addresses the first tile of the K range instead: its
+    // loads below are then unconditional like everyone's, and the compiler can count them.
+    const int g_first = left > 0 ? g0 : gbeg;
+    const u4_t *ap = p.Ap + ((int64_t)g_first * 2 * p.mblk_pad + mb0) * 64 + lane;
     auto load_a = [&](u4_t (&Aj)[MB], const u4_t *src) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) Aj[mb] = src[mb * 64];
@@ -277,7 +280,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     // fast path: first tile and first activation operands are requested before the
     // tables are built, so their latency hides behind the build
     u4_t R[4], A0[MB], A1[MB];
-    const uint8_t *tp = p.q[0] + ((int64_t)t * p.G + g0) * 4096 + lane * 16;
+    const uint8_t *tp = p.q[0] + ((int64_t)t * p.G + g_first) * 4096 + lane * 16;
     auto load_tile = [&]() {
 #pragma unroll
         for (int i = 0; i < 4; ++i) R[i] = __builtin_nontemporal_load((const u4_t *)(tp + i * 1024));
@@ -292,11 +295,14 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             row = min(row, p.lut_rows - 1);
             lutv[gl] = p.lut[0][((size_t)row << 4) + (lane & 15)];
         }
-        if (left > 0) {
-            load_tile();
-            load_a(A0, ap);
-            load_a(A1, ap + jstep);
-        }
+        // Unconditional, after the LUT row: the table build below then waits for the LUT
+        // values only, not for the first tile (a conditional load here made that wait a
+        // wait for everything).
+        __builtin_amdgcn_sched_barrier(0);
+        load_tile();
+        load_a(A0, ap);
+        load_a(A1, ap + jstep);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- pair tables ------------------------------------------------------------
@@ -405,6 +411,9 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 half_mma<4, MB, BF16, true>(Q, 0, A0, acc, lb, 8);
                 if (left > 1) ap += astep;
                 load_a(A0, ap);                           // half a tile ahead of its use
+                // issue order activations -> tile: the wait for these activations at the
+                // top of the next iteration then does not include the tile load
+                __builtin_amdgcn_sched_barrier(0);
                 stage_write();                            // next tile, requested a whole tile ago
                 if (left > 2) tp += qstep;
                 load_tile();                              // the tile after it
