@@ -74,7 +74,7 @@ def _time_graph(torch, fn, reps=3):
     return best
 
 
-def _cpu_baseline(torch, seconds_budget=20.0):
+def _cpu_baseline(torch, seconds_budget=12.0):
     """The upstream reference path as shipped (unpack the blob, gather the LUT,
     fp32 matmul; scripts/palettized_modules.py:811-824, 1241-1251 upstream) through
     the oracle, on the benchmark's first configuration: M=1, 4096 -> 4096, fp16."""
@@ -90,7 +90,8 @@ def _cpu_baseline(torch, seconds_budget=20.0):
     O.linear_reference(x, blob, lut, N, K, GS, 4)
     times = []
     t_end = time.perf_counter() + seconds_budget
-    while len(times) < 10 and (time.perf_counter() < t_end or len(times) < 3):
+    # a bounded sample: about twelve seconds of host work (at least three calls)
+    while time.perf_counter() < t_end or len(times) < 3:
         t0 = time.perf_counter()
         O.linear_reference(x, blob, lut, N, K, GS, 4)
         times.append(time.perf_counter() - t0)
