@@ -644,6 +644,7 @@ struct LaneGeom {
 template <int B>
 struct StreamRegs {
     static constexpr int kPrefetch = B == 4 ? 4 : 8;   // loads in flight per lane (a unit is 4*B bytes of it)
+    static constexpr int kEarly = B == 4 ? 1 : 2;      // loads issued ahead of the table build
     static constexpr int kEDW = 1 << (TableShape<B>::kEntryLog2 - 2);
     uint32_t q[kPrefetch][B];
     uint32_t val[kEDW];      // this thread's table entry (fast path)
@@ -670,15 +671,19 @@ __device__ __forceinline__ void stream_issue(const GemvParams &p, const GemvSeg 
     r.lane0 = (uint32_t)gm.gsub * (1024 * B) + (uint32_t)gm.cg0 * (64 * B) +
               (uint32_t)gm.l * (4 * B) + (uint32_t)gm.w * unit_bytes;
     r.step = (uint32_t)gm.nwaves * unit_bytes;
-    r.my_units = gm.units > gm.w ? (gm.units - gm.w + gm.nwaves - 1) / gm.nwaves : 0;
+    // wavefront counts, group sizes, slices per tile and table sizes are powers of two:
+    // shifts and masks instead of integer divisions throughout the prologue
+    const int nw_log2 = __builtin_ctz(gm.nwaves);
+    r.my_units = gm.units > gm.w ? (gm.units - gm.w + gm.nwaves - 1) >> nw_log2 : 0;
     const int gs = sg.gs;
-    const int ngrp_all = gs >= 128 ? 1 : 128 / gs;
-    r.grp0 = min((gm.t * 128) / gs, sg.lut_rows - 1);
+    const int gs_log2 = __builtin_ctz(gs);
+    const int ngrp_all = gs >= 128 ? 1 : 128 >> gs_log2;
+    r.grp0 = min((gm.t * 128) >> gs_log2, sg.lut_rows - 1);
     r.ngrp = min(ngrp_all, sg.lut_rows - r.grp0);
     const int items = r.ngrp * E;
     r.fast_table = items <= gm.nthreads;
     if (r.fast_table) {
-        const int item = gm.tid % items;
+        const int item = (items & (items - 1)) == 0 ? (gm.tid & (items - 1)) : gm.tid % items;
         const uint16_t *lut = st.lut + ((size_t)(r.grp0 + item / E) << B);
 #pragma unroll
         for (int s = 0; s < StreamRegs<B>::kEDW; ++s) r.val[s] = table_dword<B>(lut, item % E, s);
@@ -688,9 +693,26 @@ __device__ __forceinline__ void stream_issue(const GemvParams &p, const GemvSeg 
     // the order of use and addressed as a uniform base plus one lane-constant
     // offset: the compiler then knows how many loads are in flight at each point and
     // waits for exactly the one a unit needs.
+    // Only the first kEarly loads go out here; the rest follow the table build
+    // (stream_issue_rest).  A full batch ahead of it would put every other
+    // workgroup's activation and LUT loads behind it in the CU's memory queue.
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int n = 0; n < PF; ++n) {
+    for (int n = 0; n < StreamRegs<B>::kEarly; ++n) {
+        const uint8_t *base = n < r.my_units ? r.qrow + (size_t)n * r.step
+                                             : r.qrow - (size_t)gm.w * unit_bytes;
+        load_quarter<B>(r.q[n], uniform_ptr(base) + r.lane0);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+template <int B>
+__device__ __forceinline__ void stream_issue_rest(const LaneGeom &gm, StreamRegs<B> &r) {
+    constexpr int PF = StreamRegs<B>::kPrefetch;
+    const uint32_t unit_bytes = (uint32_t)gm.gpi * (1024 * B);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = StreamRegs<B>::kEarly; n < PF; ++n) {
         const uint8_t *base = n < r.my_units ? r.qrow + (size_t)n * r.step
                                              : r.qrow - (size_t)gm.w * unit_bytes;
         load_quarter<B>(r.q[n], uniform_ptr(base) + r.lane0);
@@ -712,12 +734,15 @@ __device__ __forceinline__ void stream_tables(const GemvStream &st, const LaneGe
     const int es = st.es;
     const int items = r.ngrp * E;
     const int nrep = 1 << (es - EL);
-    int shares = gm.nthreads / items;
+    const bool pow2 = (items & (items - 1)) == 0;   // always, unless the LUT ends inside the tile
+    const int items_log2 = 31 - __builtin_clz((unsigned)items);
+    int shares = pow2 ? gm.nthreads >> items_log2 : gm.nthreads / items;
     if (shares < 1) shares = 1;
     if (shares > nrep) shares = nrep;
-    const int per = nrep / shares;
+    const int per = pow2 ? nrep >> (31 - __builtin_clz((unsigned)shares)) : nrep / shares;
     for (int it = gm.tid; it < items * shares; it += gm.nthreads) {
-        const int item = it % items, share = it / items;
+        const int item = pow2 ? (it & (items - 1)) : it % items;
+        const int share = pow2 ? it >> items_log2 : it / items;
         const int qg = item / E, e = item % E;
         uint32_t val[EDW];
         if (r.fast_table) {
@@ -729,6 +754,20 @@ __device__ __forceinline__ void stream_tables(const GemvStream &st, const LaneGe
             for (int s = 0; s < EDW; ++s) val[s] = table_dword<B>(lut, e, s);
         }
         uint8_t *ent = lds + (size_t)qg * (E << es) + ((size_t)e << es);
+        if (es >= 4) {
+            // the replicas of an entry are contiguous: 16 bytes per store
+            uint4 pat;
+            if constexpr (EDW == 1) pat = make_uint4(val[0], val[0], val[0], val[0]);
+            else if constexpr (EDW == 2) pat = make_uint4(val[0], val[1], val[0], val[1]);
+            else pat = make_uint4(val[0], val[1], val[2], val[3]);
+            const int pieces = (per << EL) >> 4;    // 16-byte pieces of this thread's share
+            if (pieces > 0) {
+                uint8_t *mine = ent + (size_t)share * per * (1 << EL);
+                for (int k = 0; k < pieces; ++k)
+                    *(uint4 *)(mine + (((k + gm.tid) & (pieces - 1)) << 4)) = pat;
+                continue;
+            }
+        }
         for (int k = 0; k < per; ++k) {
             const int rep = share * per + ((k + gm.tid) & (per - 1));
             uint32_t *dst = (uint32_t *)(ent + (rep << EL));
@@ -753,7 +792,7 @@ __device__ __forceinline__ void stream_loop(const GemvParams &p, const GemvSeg &
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         const int row_local = (gm.cg >> 3) * 64 + v * 16;
-        int qg = gs >= 128 ? 0 : row_local / gs;
+        int qg = gs >= 128 ? 0 : row_local >> __builtin_ctz(gs);
         qg = min(qg, r.ngrp - 1);
         lane_off[v] = (uint32_t)(qg * (E << es) + ((gm.L & slot_mask) << EL));
     }
@@ -826,6 +865,7 @@ __device__ void run_stream(const GemvParams &p, const GemvSeg &sg, const GemvStr
     StreamRegs<B> r;
     stream_issue<B>(p, sg, st, gm, r);
     stream_tables<B>(st, gm, lds, r);
+    stream_issue_rest<B>(gm, r);
     __syncthreads();
     stream_loop<B, BF16>(p, sg, st, gm, lds, r, acc);
     __syncthreads();
@@ -888,12 +928,13 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     const int rw = lpg >> 1;                        // rows per workgroup
     const int spt = 128 / rw;                       // row slices per tile
     const int sl = (int)blockIdx.x - sg.col0;
-    gm.t = sl / spt;
-    gm.cg0 = (sl % spt) * (rw >> 3);
+    const int spt_log2 = 8 - p.lpg_log2;            // spt = 128 / rw = 256 >> lpg_log2
+    gm.t = sl >> spt_log2;
+    gm.cg0 = (sl & (spt - 1)) * (rw >> 3);
     gm.cg = gm.cg0 + (gm.l >> 4);
     const int s = blockIdx.y;
     gm.g_lo = s * p.gs_tiles;
-    gm.units = p.gs_tiles / gm.gpi;
+    gm.units = p.gs_tiles >> (6 - p.lpg_log2);      // gpi = 64 >> lpg_log2
     const int k0 = gm.g_lo * 64, kc = p.gs_tiles * 64;
 
     float *red = (float *)(lds + p.lds_red);        // [2][nwaves][32] row sums
@@ -954,6 +995,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
             if (BFIX != 0 && so == 0 && si == 0) {
                 if constexpr (BFIX != 0) {
                     stream_tables<BF>(st, gm, lds, first);
+                    stream_issue_rest<BF>(gm, first);
                     __syncthreads();
                     FLUTE_TRACE(3);
                     stream_loop<BF, BF16>(p, og, st, gm, lds, first, acc);
