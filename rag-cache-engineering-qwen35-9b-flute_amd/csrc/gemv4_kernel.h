@@ -398,6 +398,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 ws_store(p.P + (size_t)s * p.p_stride + kp->seg[so == 1 ? 1 : si0].n0 + n, yv[so]);
             }
         }
+        ws_stores_done();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (tid == 0) {

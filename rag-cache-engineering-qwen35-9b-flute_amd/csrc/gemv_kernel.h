@@ -130,6 +130,10 @@ __device__ __forceinline__ void ws_store(float *p, float v) {
 __device__ __forceinline__ float ws_load(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// A store is visible device-wide once it has been acknowledged; the ticket that
+// announces the stores of a workgroup may only be taken after that.  (A barrier does
+// not wait for outstanding memory operations.)
+__device__ __forceinline__ void ws_stores_done() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
 
 // Sum over the 16 lanes of a DPP row; every lane of the row ends with the total.
 __device__ __forceinline__ float row16_sum(float v) {
@@ -1052,6 +1056,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
             }
         }
         // the stores are acknowledged by the device-coherent level before the ticket
+        ws_stores_done();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (gm.tid == 0) {
