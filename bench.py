@@ -109,18 +109,19 @@ def _gemv_section(torch, _lib, ctypes, sets, gen, dev, O):
     """The other M = 1 configurations beside the headline block, each parity-gated against
     the oracle on the rows of one tile: the north-star GEMV 4096 -> 12288 (GB/s on packed
     index + LUT bytes, the numerator the target is stated on), the same GEMV with the
-    block-128 Hadamard rotation fused into its prologue, and the narrow split-K shapes."""
+    block-128 Hadamard rotation fused into its prologue, and the narrow shapes of the split-K
+    configuration."""
     out = {}
     act = torch.bfloat16
     x = torch.randn(1, H, device=dev, generator=gen).to(act)
     stream = lambda: torch.cuda.current_stream().cuda_stream
 
-    def run(name, descs, N, K, xin, keep, signs=None, block=0):
+    def run(name, descs, N, K, xin, keep, signs=None, block=0, split=0):
         y = torch.zeros(1, N, dtype=act, device=dev)
 
         def call(i):
             st = _lib.lib.flute_gemv(ctypes.byref(descs[i % len(descs)]), xin.data_ptr(),
-                                     y.data_ptr(), _lib.BF16, 0, stream())
+                                     y.data_ptr(), _lib.BF16, split, stream())
             if st != 0:
                 raise RuntimeError(_lib.last_error())
 
@@ -139,7 +140,7 @@ def _gemv_section(torch, _lib, ctypes, sets, gen, dev, O):
         err = float(((got - ref) ** 2).sum() / (ref ** 2).sum()) ** 0.5
         if err > 4e-3:
             raise SystemExit(f"bench.py: parity gate failed for {name} ({err:.2e})")
-        n = 96
+        n = max(96, len(descs))                     # every weight of the rotation once per replay
         us = _time_graph(torch, lambda: [call(i) for i in range(n)]) / n * 1e3
         wbytes = N * K // 2 + (N // GS) * 32
         out[name] = {"us_per_call": round(us, 2), "gbs_index_plus_lut": round(wbytes / us / 1e3, 1),
@@ -166,9 +167,23 @@ def _gemv_section(torch, _lib, ctypes, sets, gen, dev, O):
         d.signs, d.rot_block = signs.data_ptr(), 128
         rot.append(d)
     run("gemv_4096x12288_fht128_fused", rot, I, H, x, keep, signs=signs, block=128)
+    # narrow outputs: the library's own choice (it does not split K on this device) and the
+    # forced K splits of the configuration beside it; enough weights to stay out of the caches
     for N in (1024, 512):
-        ws = [_weights(torch, N, H, gen, dev, torch.float16) for _ in range(16)]
-        run(f"gemv_split_k_4096x{N}", [_desc(_lib, b, l, N, H) for b, l in ws], N, H, x, ws)
+        count = int(3.1 * 256 * 2 ** 20 // (N * H // 2)) + 1
+        ws = [_weights(torch, N, H, gen, dev, torch.float16) for _ in range(count)]
+        ds = [_desc(_lib, b, l, N, H) for b, l in ws]
+        name = f"gemv_narrow_4096x{N}"
+        run(name, ds, N, H, x, ws)
+        res = out[name]
+        res["split_chosen"] = int(_lib.lib.flute_pick_split(N, H))
+        res["weights_in_rotation"] = count
+        sweep = {}
+        for sp in (2, 4, 8):
+            run("_sweep", ds, N, H, x, ws, split=sp)
+            sweep[str(sp)] = out.pop("_sweep")["us_per_call"]
+        res["us_per_call_forced_split"] = sweep
+        del ws, ds
     return out
 
 

@@ -188,7 +188,9 @@ flute_status flute_embedding(const flute_linear *w, const int64_t *ids, int64_t 
 
 /*
  * The K-split the library would choose for an (N, K) GEMV on this device
- * (the MI355X restatement of gemv_pick_split, src/gemv_host.cpp:29-38).
+ * (the MI355X counterpart of gemv_pick_split, src/gemv_host.cpp:29-38).  On this
+ * device the unsplit launch measured fastest for every shape, so the answer is 1;
+ * callers that pass an explicit split to flute_gemv still get it.
  * Pure host arithmetic: usable without a GPU.
  */
 int flute_pick_split(int N, int K);

@@ -44,11 +44,13 @@ struct Plan {
 };
 
 // Shape of the launch for `rows` output rows over G tiles of K.  A workgroup
-// owns `rw` rows; without a K split nothing is exchanged between workgroups, so
-// the split stays 1 as long as the row slices alone give every CU at least two
-// workgroups.
+// owns `rw` rows.  The library's own policy never splits K: the exchange between
+// workgroups (partial sums written through, a ticket, the last arrival reading them
+// back) is three memory round trips, about 1.5 us, and measured slower than the
+// unsplit launch with eight wavefronts for every narrow shape tried (N = 128...3072
+// at K = 2048...16384; e.g. N = 1024, K = 4096: 5.0 us against 6.7 us split four
+// ways).  A caller's explicit split is honoured.
 void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *waves) {
-    bool exact_tiling = false;
     int best_rw = env_int("FLUTE_GEMV_RW", 0);
     if (best_rw != 8 && best_rw != 16 && best_rw != 32) {
         best_rw = 8;
@@ -61,7 +63,6 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
         // 9.5 us for 768 with a three-way K split).
         if (rows % (16 * kNumCU) == 0 && rows / (16 * kNumCU) <= 2 && G / 2 >= 64) {
             best_rw = 16;
-            exact_tiling = true;
         }
     }
     int sp = split_req;
@@ -71,33 +72,20 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
         while (G % sp == 0 && (G / sp) % (32 / best_rw) != 0 && best_rw < 32) best_rw *= 2;
     } else {
         sp = 1;
-        const long slices = rows / best_rw;
-        const int gpi = 32 / best_rw;
-        if (slices < 2 * kNumCU && !exact_tiling) {
-            // narrow output: split K until the grid reaches about three workgroups per CU
-            long best_cost = -1;
-            for (int d = 1; d <= G; ++d) {
-                if (G % d || (G / d) % gpi) continue;
-                if (G / d < 4 * gpi && d > 1) continue;
-                const long wgs = slices * d;
-                const long target = 3 * kNumCU;
-                const long cost = wgs > target ? 2 * (wgs - target) : target - wgs;
-                if (best_cost < 0 || cost < best_cost) { best_cost = cost; sp = d; }
-            }
-        }
         while ((G / sp) % (32 / best_rw) != 0 && best_rw < 32) best_rw *= 2;
     }
     *rw = best_rw;
     *split = sp;
     int wv = env_int("FLUTE_GEMV_WAVES", 0);
     if (wv != 1 && wv != 2 && wv != 4 && wv != 8) {
-        // four wavefronts with eight loads each in flight measured best; eight when a
-        // workgroup has a long K range to itself and the grid is small enough for all
-        // of it to be resident at once with eight (two workgroups per CU)
+        // Eight wavefronts when the whole grid is resident with eight (two workgroups per
+        // CU) and each wavefront still has two loads or more; short K ranges (fewer than
+        // four loads per wavefront at eight) only up to one workgroup per CU.  Otherwise
+        // four, fewer for very short K.
         const int units = (G / sp) / (32 / best_rw);
         const long wgs = (long)(rows / best_rw) * sp;
-        wv = (units >= 64 && wgs <= 2 * kNumCU) ? 8
-                                                : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
+        const bool eight = units >= 16 && wgs <= 2 * kNumCU && (units >= 32 || wgs <= kNumCU);
+        wv = eight ? 8 : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
     }
     *waves = wv;
 }

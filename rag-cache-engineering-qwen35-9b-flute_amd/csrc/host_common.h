@@ -12,7 +12,6 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who);
 
 // K-split the GEMV launchers use for `tiles` 128-row workgroup columns over
 // G = K/64 tiles of K.
-int pick_split_tiles(int tiles, int G);
 
 // Split-K workspace of the current device: `floats` fp32 partial sums and
 // `ints` zero-initialised tickets.  Grows geometrically, never shrinks; the

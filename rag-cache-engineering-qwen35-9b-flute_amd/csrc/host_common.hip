@@ -79,26 +79,6 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who) {
     return FLUTE_OK;
 }
 
-// One workgroup holds a 64 KB table, so two fit a CU; three waves of 256
-// workgroups keep every CU busy while the tail of one wave drains.
-int pick_split_tiles(int tiles, int G) {
-    if (tiles <= 0 || G <= 0) return 1;
-    const int target = 3 * kNumCU;
-    int best = 1;
-    long best_cost = -1;
-    for (int d = 1; d <= G; ++d) {
-        if (G % d) continue;
-        if (G / d < 2 && d > 1) continue;          // keep two 64-k tiles per workgroup
-        const long wgs = (long)tiles * d;
-        const long cost = wgs > target ? (wgs - target) * 2 : (target - wgs);
-        if (best_cost < 0 || cost < best_cost) {
-            best_cost = cost;
-            best = d;
-        }
-    }
-    return best;
-}
-
 struct Workspace {
     float *P = nullptr;
     int *tickets = nullptr;
