@@ -175,8 +175,16 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     const int64_t units = (int64_t)tiles * mchunks;
     p.mblk_pad = mchunks * shape.mb * shape.mw;
     const int64_t cap = (int64_t)kNumCU * shape.wg_per_cu;
+    // K is split until the grid reaches one workgroup per CU, while every wavefront keeps
+    // two tiles or more; with four blocks of rows per wavefront at most four ways, because
+    // the workgroup that arrives last reads every 32 KB partial tile of its unit back
+    // (measured at M = 64: 12288 -> 4096 29.7 us four ways, 36.4 us eight ways; 4096 -> 4096
+    // 21.8 us four ways, 23.0 us two ways, 24.6 us eight ways).
+    const int max_split = shape.mb == 1 ? 64 : 4;
     int ksplit = 1;
-    while (units * ksplit * 2 <= cap && p.G / (ksplit * 2) >= shape.kw) ksplit *= 2;
+    while (units * ksplit * 2 <= cap && ksplit * 2 <= max_split &&
+           p.G / (ksplit * 2) >= shape.kw * 2)
+        ksplit *= 2;
     if (const char *e = getenv("FLUTE_GEMM_KSPLIT")) {
         const int v = atoi(e);
         if (v >= 1 && v <= p.G) ksplit = v;
