@@ -53,9 +53,13 @@ struct Plan {
 void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *waves) {
     int best_rw = env_int("FLUTE_GEMV_RW", 0);
     if (best_rw != 8 && best_rw != 16 && best_rw != 32) {
-        best_rw = 8;
-        for (int cand : {32, 16, 8}) {
-            if (rows / cand >= 2 * kNumCU + kNumCU / 2) { best_rw = cand; break; }
+        // The narrowest slices whose grid is still resident at once (three four-wavefront
+        // workgroups per CU): a second round of workgroups costs far more than wider
+        // slices do (8192 rows at K = 4096: 512 sixteen-row workgroups 7.3 us, 1024
+        // eight-row ones 13.2 us; 16384 rows: 11.3 us with 32 rows against 15.3 with 16).
+        best_rw = 32;
+        for (int cand : {8, 16}) {
+            if (rows / cand <= 3 * kNumCU) { best_rw = cand; break; }
         }
         // A grid of exactly one or two 16-row workgroups per CU, unsplit, measured best
         // where K is long enough to give each of them eight wavefronts (4096 rows at
@@ -78,13 +82,14 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
     *split = sp;
     int wv = env_int("FLUTE_GEMV_WAVES", 0);
     if (wv != 1 && wv != 2 && wv != 4 && wv != 8) {
-        // Eight wavefronts when the whole grid is resident with eight (two workgroups per
-        // CU) and each wavefront still has two loads or more; short K ranges (fewer than
-        // four loads per wavefront at eight) only up to one workgroup per CU.  Otherwise
-        // four, fewer for very short K.
+        // Eight wavefronts when each still has two loads or more and the grid is at most
+        // one workgroup per CU, or two per CU of eight-row workgroups with a long K range
+        // (measured: 384 eight-row workgroups at K >= 8192 gain 2-10 % from eight, 512
+        // sixteen- or 32-row ones lose 3-8 %).  Otherwise four, fewer for very short K.
         const int units = (G / sp) / (32 / best_rw);
         const long wgs = (long)(rows / best_rw) * sp;
-        const bool eight = units >= 16 && wgs <= 2 * kNumCU && (units >= 32 || wgs <= kNumCU);
+        const bool eight = units >= 16 && (wgs <= kNumCU || (wgs <= 2 * kNumCU && units >= 32 &&
+                                                             best_rw == 8));
         wv = eight ? 8 : (units >= 4 ? 4 : (units >= 2 ? 2 : 1));
     }
     *waves = wv;
