@@ -14,13 +14,28 @@ struct GemmShape {
     int wg_per_cu;        // workgroups the policy expects to be resident per CU
 };
 
-// M <= 16: one block, eight k ways (the launch is a weight stream, like the GEMV).
-// Otherwise four blocks per wavefront: 64 rows of A per workgroup with eight k ways
-// while that still fits the device in one round of workgroups, else 128 rows (two m
-// groups, four k ways); further rows go to gridDim.y.  The tables plus staging take
-// most of a CU's LDS, so one workgroup per CU is resident.
-GemmShape choose_gemm_shape(int M, int tiles) {
+// One 16-row block per wavefront and eight k ways (the launch is a weight stream, like
+// the GEMV) for M <= 16, and for larger M as long as one workgroup per 16 rows and tile
+// still fits the device in one round and the weights are not re-read too often (every
+// 16-row chunk streams its tile's indices again): measured at M = 32, 4096 -> 12288
+// 17.9 us against 24.6 us with 64-row workgroups; M = 128, 4096 -> 4096 18.9 against
+// 24.9 us; beyond 100 MB of index traffic the 64-row shape wins (M = 96, 12288 -> 4096).
+// Otherwise four blocks per wavefront: 64 rows of A per workgroup with eight k ways while
+// that still fits the device in one round, else 128 rows (two m groups, four k ways);
+// further rows go to gridDim.y.  The tables plus staging take most of a CU's LDS, so one
+// workgroup per CU is resident.  FLUTE_GEMM_ROWS = 16, 64 or 128 forces the rows of A per
+// workgroup (a tuning and test knob, like FLUTE_GEMV_RW).
+GemmShape choose_gemm_shape(int M, int tiles, int64_t index_bytes) {
+    if (const char *e = getenv("FLUTE_GEMM_ROWS")) {
+        const int v = atoi(e);
+        if (v == 16) return {1, 8, 1, 1};
+        if (v == 64) return {4, 8, 1, 1};
+        if (v == 128) return {4, 4, 2, 1};
+    }
     if (M <= 16) return {1, 8, 1, 1};
+    const int chunks16 = (M + 15) / 16;
+    if ((int64_t)tiles * chunks16 <= kNumCU && chunks16 * index_bytes <= (int64_t)100 << 20)
+        return {1, 8, 1, 1};
     const int chunks64 = (M + 63) / 64;
     if ((int64_t)tiles * chunks64 <= kNumCU) return {4, 8, 1, 1};
     return {4, 4, 2, 1};
@@ -145,7 +160,7 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
                   M, w->R);
     hipStream_t stream = (hipStream_t)stream_;
 
-    GemmShape shape = choose_gemm_shape(M, w->N / 128);
+    GemmShape shape = choose_gemm_shape(M, w->N / 128, w->q1_bytes + (w->b2 > 0 ? w->q2_bytes : 0));
     GemmParams p = {};
     p.nstreams = w->b2 > 0 ? 2 : 1;
     p.q[0] = (const uint8_t *)w->q1;

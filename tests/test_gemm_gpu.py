@@ -68,6 +68,33 @@ def test_gemm_single_stream_fp16(M, N, K, bits, gs):
     assert torch.equal(y, y2)                           # deterministic
 
 
+@pytest.mark.parametrize("rows", ["16", "64", "128"])
+@pytest.mark.parametrize("M,N,K,bits,gs", [c for c in SINGLE if c[0] > 16])
+def test_gemm_every_workgroup_shape(monkeypatch, rows, M, N, K, bits, gs):
+    """The library picks the rows of A per workgroup (16, 64 or 128) from M, N and K; at
+    the small N of these cases it would always pick 16, so each shape is forced in turn
+    (FLUTE_GEMM_ROWS, read per call) and must give the oracle's result."""
+    monkeypatch.setenv("FLUTE_GEMM_ROWS", rows)
+    w = make_weight(N, K, bits, gs, seed=M + N + K + bits, device=DEV)
+    x = make_x(M, K, seed=11)
+    y = fx.qgemm_per_group_lut(x.to(DEV), w["blob_d"], w["lut_d"], bitwidth=bits, group_size=gs,
+                               indices_layout=f"idx{bits}").cpu()
+    assert rel_l2(y, _exact(w, x).half()) <= TOL
+
+
+@pytest.mark.parametrize("rows", ["16", "64", "128"])
+def test_gemm_two_streams_residual_bias_every_workgroup_shape(monkeypatch, rows):
+    monkeypatch.setenv("FLUTE_GEMM_ROWS", rows)
+    M, N, K = 40, 256, 1024
+    for lut_dtype, act_dtype in ((torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16)):
+        w = make_weight(N, K, 4, 128, seed=7, bits2=2, rank=8, bias=True, lut_dtype=lut_dtype,
+                        act_dtype=act_dtype, device=DEV)
+        x = make_x(M, K, seed=13, dtype=act_dtype)
+        y = _dual(w, x).cpu()
+        ref = _exact(w, x.to(lut_dtype)).to(act_dtype)
+        assert rel_l2(y, ref) <= (TOL if act_dtype == torch.float16 else TOL_BF16)
+
+
 DUAL = [
     # M, N, K, bits, gs, bits2, rank, bias
     (8, 512, 1024, 4, 128, 1, 0, False),
