@@ -14,28 +14,32 @@ struct GemmShape {
     int wg_per_cu;        // workgroups the policy expects to be resident per CU
 };
 
-// One 16-row block per wavefront and eight k ways (the launch is a weight stream, like
-// the GEMV) for M <= 16, and for larger M as long as one workgroup per 16 rows and tile
-// still fits the device in one round and the weights are not re-read too often (every
-// 16-row chunk streams its tile's indices again): measured at M = 32, 4096 -> 12288
-// 17.9 us against 24.6 us with 64-row workgroups; M = 128, 4096 -> 4096 18.9 against
-// 24.9 us; beyond 100 MB of index traffic the 64-row shape wins (M = 96, 12288 -> 4096).
-// Otherwise four blocks per wavefront: 64 rows of A per workgroup with eight k ways while
-// that still fits the device in one round, else 128 rows (two m groups, four k ways);
-// further rows go to gridDim.y.  The tables plus staging take most of a CU's LDS, so one
-// workgroup per CU is resident.  FLUTE_GEMM_ROWS = 16, 64 or 128 forces the rows of A per
-// workgroup (a tuning and test knob, like FLUTE_GEMV_RW).
+// Rows of A per workgroup.  One or two 16-row blocks per wavefront with eight k ways (the
+// launch is then a weight stream, like the GEMV) as long as one workgroup per 16 (32) rows
+// and tile fits the device in one round and the indices are not re-read too often: every
+// chunk of rows streams its tile again, and beyond about 64 MB (100 MB) of index traffic
+// the next shape wins.  Measured: M = 32, 4096 -> 12288: 18.0 us with 16 rows, 24.6 us
+// with 64; M = 64: 21.5 us with 32 rows, 26.0 us with 64; M = 256, 4096 -> 4096: 23.8 us
+// with 32 rows, 29.0 us with 64; M = 96, 12288 -> 4096: 31.6 us with 32 rows, 37.8 us
+// with 16, 34.7 us with 64.  Otherwise four blocks per wavefront: 64 rows per workgroup
+// with eight k ways while that fits the device in one round, else 128 rows (two m groups,
+// four k ways); further rows go to gridDim.y.  The tables plus staging take most of a
+// CU's LDS, so one workgroup per CU is resident.  FLUTE_GEMM_ROWS = 16, 32, 64 or 128
+// forces the shape (a tuning and test knob, like FLUTE_GEMV_RW).
 GemmShape choose_gemm_shape(int M, int tiles, int64_t index_bytes) {
     if (const char *e = getenv("FLUTE_GEMM_ROWS")) {
         const int v = atoi(e);
         if (v == 16) return {1, 8, 1, 1};
+        if (v == 32) return {2, 8, 1, 1};
         if (v == 64) return {4, 8, 1, 1};
         if (v == 128) return {4, 4, 2, 1};
     }
     if (M <= 16) return {1, 8, 1, 1};
-    const int chunks16 = (M + 15) / 16;
-    if ((int64_t)tiles * chunks16 <= kNumCU && chunks16 * index_bytes <= (int64_t)100 << 20)
+    const int chunks16 = (M + 15) / 16, chunks32 = (M + 31) / 32;
+    if ((int64_t)tiles * chunks16 <= kNumCU && chunks16 * index_bytes <= (int64_t)64 << 20)
         return {1, 8, 1, 1};
+    if ((int64_t)tiles * chunks32 <= kNumCU && chunks32 * index_bytes <= (int64_t)100 << 20)
+        return {2, 8, 1, 1};
     const int chunks64 = (M + 63) / 64;
     if ((int64_t)tiles * chunks64 <= kNumCU) return {4, 8, 1, 1};
     return {4, 4, 2, 1};
@@ -63,6 +67,7 @@ flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 gri
                                hipStream_t stream) {
     if (!BF16 && p.nstreams == 1 && p.bits[0] == 4 && p.rep_log2[0] == 6) {
         if (s.mb == 1) return launch_gemm<1, 8, 1, false, 4, true>(p, grid, lds, stream);
+        if (s.mb == 2) return launch_gemm<2, 8, 1, false, 4, true>(p, grid, lds, stream);
         if (s.mw == 1) return launch_gemm<4, 8, 1, false, 4, true>(p, grid, lds, stream);
         return launch_gemm<4, 4, 2, false, 4, true>(p, grid, lds, stream);
     }
@@ -94,6 +99,7 @@ template <bool BF16>
 flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 grid, int lds,
                                hipStream_t stream) {
     if (s.mb == 1) return launch_gemm_bits<1, 8, 1, BF16>(p, grid, lds, stream);
+    if (s.mb == 2) return launch_gemm_bits<2, 8, 1, BF16>(p, grid, lds, stream);
     if (s.mw == 1) return launch_gemm_bits<4, 8, 1, BF16>(p, grid, lds, stream);
     return launch_gemm_bits<4, 4, 2, BF16>(p, grid, lds, stream);
 }

@@ -68,10 +68,10 @@ def test_gemm_single_stream_fp16(M, N, K, bits, gs):
     assert torch.equal(y, y2)                           # deterministic
 
 
-@pytest.mark.parametrize("rows", ["16", "64", "128"])
+@pytest.mark.parametrize("rows", ["16", "32", "64", "128"])
 @pytest.mark.parametrize("M,N,K,bits,gs", [c for c in SINGLE if c[0] > 16])
 def test_gemm_every_workgroup_shape(monkeypatch, rows, M, N, K, bits, gs):
-    """The library picks the rows of A per workgroup (16, 64 or 128) from M, N and K; at
+    """The library picks the rows of A per workgroup (16, 32, 64 or 128) from M, N and K; at
     the small N of these cases it would always pick 16, so each shape is forced in turn
     (FLUTE_GEMM_ROWS, read per call) and must give the oracle's result."""
     monkeypatch.setenv("FLUTE_GEMM_ROWS", rows)
@@ -82,7 +82,7 @@ def test_gemm_every_workgroup_shape(monkeypatch, rows, M, N, K, bits, gs):
     assert rel_l2(y, _exact(w, x).half()) <= TOL
 
 
-@pytest.mark.parametrize("rows", ["16", "64", "128"])
+@pytest.mark.parametrize("rows", ["16", "32", "64", "128"])
 def test_gemm_two_streams_residual_bias_every_workgroup_shape(monkeypatch, rows):
     monkeypatch.setenv("FLUTE_GEMM_ROWS", rows)
     M, N, K = 40, 256, 1024
