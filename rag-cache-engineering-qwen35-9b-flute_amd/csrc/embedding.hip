@@ -9,6 +9,8 @@
 #include "fht_dev.h"
 #include "host_common.h"
 
+#include <atomic>
+
 namespace flute {
 
 namespace {
@@ -180,7 +182,7 @@ extern "C" flute_status flute_embedding(const flute_linear *w, const int64_t *id
         } else {
             lds = (size_t)make_segments(w->K, 0).len[0] * 4;
         }
-        static bool attr_done = false;
+        static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
         if (!attr_done) {
             FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)embedding_kernel,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 65536));

@@ -3,6 +3,8 @@
 #include "fht_dev.h"
 #include "host_common.h"
 
+#include <atomic>
+
 #include <cmath>
 
 namespace flute {
@@ -140,7 +142,7 @@ extern "C" flute_status flute_fht(const void *x, const float *signs, const float
         lds_bytes = (size_t)segs.len[0] * 4;
     }
     if (M == 0) return FLUTE_OK;
-    static bool attr_done = false;
+    static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
         FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)fht_kernel,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 65536));

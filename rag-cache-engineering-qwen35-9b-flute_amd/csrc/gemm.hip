@@ -5,6 +5,8 @@
 #include "gemm_kernel.h"
 #include "host_common.h"
 
+#include <atomic>
+
 namespace flute {
 
 namespace {
@@ -47,7 +49,7 @@ GemmShape choose_gemm_shape(int M, int tiles, int64_t index_bytes) {
 
 template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false>
 flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
-    static bool attr_done = false;
+    static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
         FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1, PERM>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,

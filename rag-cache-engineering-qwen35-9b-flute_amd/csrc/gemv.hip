@@ -4,6 +4,8 @@
 #include "gemv4_kernel.h"
 #include "host_common.h"
 
+#include <atomic>
+
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -275,7 +277,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
 
 template <bool BF16, int BFIX>
 flute_status launch_typed(Plan &plan, hipStream_t stream) {
-    static bool attr_done = false;
+    static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
         FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv_kernel<BF16, BFIX>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -297,7 +299,7 @@ flute_status launch_typed(Plan &plan, hipStream_t stream) {
 
 template <int LPGL, int NW, int PF, bool BF16>
 flute_status launch_fast4(Plan &plan, hipStream_t stream) {
-    static bool attr_done = false;
+    static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
         FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv4_kernel<LPGL, NW, PF, BF16>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
