@@ -18,11 +18,20 @@ struct FhtParams {
     void *out;
     const float *signs;
     const float *awq;
+    int64_t ldx, ldo;   // row strides of x and out in elements
     int K;
     int dtype;      // flute_dtype of x and out
     int adjoint;
     int block;      // > 0: equal blocks
     int chunk;      // columns transformed per pass in block mode
+    // Operand-order output for the LUT GEMM instead of rows (ap != NULL): the rotated row
+    // m is rounded to `dtype`, converted to the LUT's 16-bit type and written where the
+    // GEMM's activation pre-pass would put it, Ap[g][j][m / 16][lane][8]; rows from M up
+    // to the padded count are written as zeros.
+    uint32_t *ap;
+    int ap_M, ap_mblk_pad, ap_bf16;
+    int vec_io;     // x and out rows allow 16-byte accesses (16-bit types only)
+    int vec_mul;    // signs and awq allow 16-byte loads
 };
 
 __device__ __forceinline__ float load_any(const void *p, int64_t i, int dtype) {
@@ -36,11 +45,145 @@ __device__ __forceinline__ void store_any(void *p, int64_t i, int dtype, float v
 
 // forward:  out = ((x [*awq]) @ H) * signs * inv [/ awq]   (fht.py:206-222, 646-651 upstream)
 // adjoint:  out = ((x * signs) @ H) * inv                  (fht.py:225-238 upstream)
+// Eight consecutive columns k0...k0+7 (k0 a multiple of 8) of row m in operand order:
+// k = g*64 + (2j + ktl)*16 + 2*kg + 8*s2 + e lives in lane kg*16 + m%16 of block m/16,
+// dword ktl*2 + s2, half e; so the eight values are the (e = 0, 1) pairs of the four
+// lanes kg = 0...3 at one dword position.
+__device__ __forceinline__ void store_operand_order(const FhtParams &p, int m, int k0,
+                                                    const uint16_t (&v)[8]) {
+    const int g = k0 >> 6, kl = k0 & 63;
+    const int jh = kl >> 5, s = ((kl >> 4) & 1) * 2 + ((kl >> 3) & 1);
+    const int64_t unit = ((int64_t)(g * 2 + jh) * p.ap_mblk_pad + (m >> 4)) * 64 + (m & 15);
+#pragma unroll
+    for (int kg = 0; kg < 4; ++kg)
+        p.ap[(unit + kg * 16) * 4 + s] = (uint32_t)v[2 * kg] | ((uint32_t)v[2 * kg + 1] << 16);
+}
+
+__device__ __forceinline__ void load_mul8(const float *m, int k, int vec, float (&v)[8]) {
+    if (vec) {
+        const float4 a = *(const float4 *)(m + k), b = *(const float4 *)(m + k + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[q] = m[k + q];
+    }
+}
+
+// Equal blocks of at most 256 columns without the LDS buffer.  A thread holds eight
+// consecutive columns: the stages of length 1, 2, 4 are butterflies between its own
+// registers, the stages of length 8 ... block/2 pair it with the lane whose number differs
+// in one bit (ds_swizzle: the LDS crossbar, no memory access).  The lower lane of a pair
+// keeps a + b and the upper a - b, formed as fma(mine, +-1, other): the product is exact,
+// so every value sees the same single rounding per stage, in the same ascending order, as
+// in the buffered butterfly, and the result is bit-identical to it.  One memory round
+// trip, no barrier.  The lanes of a block are always in the same step of the loop
+// (a step covers 2048 columns, a multiple of every block), so a lane's partners are active.
+__device__ __forceinline__ void fht_blocks_inwave(const FhtParams &p, int64_t row, int64_t orow,
+                                                  int tid) {
+    const int nst = 31 - __builtin_clz((unsigned)p.block);
+    const float inv = inv_sqrt_pow2(nst);
+    const int lane = tid & 63;
+    const int pair_lanes = p.block >> 3;               // lanes of one block: 4 ... 32
+    const int bf16 = p.dtype == FLUTE_BF16;
+    for (int j = tid * 8; j < p.K; j += kFhtThreads * 8) {
+        float f[8], sg[8], sc[8];
+        if (p.vec_io) {
+            const uint4 raw = *(const uint4 *)((const uint16_t *)p.x + row + j);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const uint16_t h = (uint16_t)(w[q >> 1] >> (16 * (q & 1)));
+                f[q] = bf16 ? bf2f(h) : h2f(h);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) f[q] = load_any(p.x, row + j + q, p.dtype);
+        }
+        load_mul8(p.signs, j, p.vec_mul, sg);
+        if (p.awq) load_mul8(p.awq, j, p.vec_mul, sc);
+        if (p.adjoint || p.awq) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) f[q] *= p.adjoint ? sg[q] : sc[q];
+        }
+#pragma unroll
+        for (int len = 1; len < 8; len <<= 1) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                if ((q & len) == 0) {
+                    const float a = f[q], c = f[q | len];
+                    f[q] = a + c;
+                    f[q | len] = a - c;
+                }
+            }
+        }
+        // and_mask 0x1f, or_mask 0, xor_mask m: lane ^ m inside each half of the wavefront
+#define FLUTE_XOR_STAGE(m)                                                                   \
+        if (pair_lanes > (m)) {                                                              \
+            const float sgn = (lane & (m)) ? -1.0f : 1.0f;                                   \
+            _Pragma("unroll") for (int q = 0; q < 8; ++q) {                                  \
+                const float other = __int_as_float(__builtin_amdgcn_ds_swizzle(              \
+                    __float_as_int(f[q]), ((m) << 10) | 0x1f));                              \
+                f[q] = fmaf(f[q], sgn, other);                                               \
+            }                                                                                \
+        }
+        FLUTE_XOR_STAGE(1)
+        FLUTE_XOR_STAGE(2)
+        FLUTE_XOR_STAGE(4)
+        FLUTE_XOR_STAGE(8)
+        FLUTE_XOR_STAGE(16)
+#undef FLUTE_XOR_STAGE
+        uint16_t op[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            float t;
+            if (p.adjoint) {
+                t = f[q] * inv;
+            } else {
+                t = f[q] * sg[q] * inv;
+                if (p.awq) t = t / sc[q];
+            }
+            f[q] = t;
+            if (p.dtype != FLUTE_F32) {
+                uint16_t a = round_act(t, bf16);
+                if (p.ap && bf16 != p.ap_bf16) a = round_act(bf16 ? bf2f(a) : h2f(a), p.ap_bf16);
+                op[q] = a;
+            }
+        }
+        if (p.ap) {
+            store_operand_order(p, blockIdx.x, j, op);
+        } else if (p.dtype == FLUTE_F32) {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) ((float *)p.out)[orow + j + q] = f[q];
+        } else if (p.vec_io) {
+            *(uint4 *)((uint16_t *)p.out + orow + j) =
+                make_uint4((uint32_t)op[0] | ((uint32_t)op[1] << 16),
+                           (uint32_t)op[2] | ((uint32_t)op[3] << 16),
+                           (uint32_t)op[4] | ((uint32_t)op[5] << 16),
+                           (uint32_t)op[6] | ((uint32_t)op[7] << 16));
+        } else {
+#pragma unroll
+            for (int q = 0; q < 8; ++q) ((uint16_t *)p.out)[orow + j + q] = op[q];
+        }
+    }
+}
+
 __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     float *buf = (float *)lds;
     const int tid = threadIdx.x;
-    const int64_t row = (int64_t)blockIdx.x * p.K;
+    const int64_t row = (int64_t)blockIdx.x * p.ldx;
+    const int64_t orow = (int64_t)blockIdx.x * p.ldo;
+    if (p.ap && (int)blockIdx.x >= p.ap_M) {           // padding row of the operand image
+        const uint16_t zero[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int j = tid * 8; j < p.K; j += kFhtThreads * 8)
+            store_operand_order(p, blockIdx.x, j, zero);
+        return;
+    }
+    if (p.block > 0 && p.block <= 256) {
+        fht_blocks_inwave(p, row, orow, tid);
+        return;
+    }
     // block mode: chunks of whole blocks; otherwise the descending power-of-two
     // segments of K (fht.py:118-134 upstream)
     for (int off = 0; off < p.K;) {
@@ -53,6 +196,21 @@ __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
             count = 1 << nstages;
         }
         const float inv = inv_sqrt_pow2(nstages);
+        // The output multipliers of a thread's first two steps are requested together
+        // with the row, so the output phase does not start with a memory round trip.
+        const int j0 = tid * 8, j1 = j0 + kFhtThreads * 8;
+        float sg0[8], sg1[8], sc0[8], sc1[8];
+        auto load_mul = [&](int j, float (&sg)[8], float (&sc)[8]) {
+            if (p.adjoint) return;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) sg[q] = p.signs[off + j + q];
+            if (p.awq) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) sc[q] = p.awq[off + j + q];
+            }
+        };
+        if (j0 < count) load_mul(j0, sg0, sc0);
+        if (j1 < count) load_mul(j1, sg1, sc1);
         // Eight columns per thread and step; the loads of a step (row, signs, scale) are
         // independent and issued together, so each phase is one memory round trip.
 #pragma unroll 2
@@ -72,17 +230,8 @@ __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
         }
         __syncthreads();
         fht_lds(buf, count, nstages, tid, kFhtThreads);
-#pragma unroll 2
-        for (int j = tid * 8; j < count; j += kFhtThreads * 8) {
-            float sg[8], sc[8];
-            if (!p.adjoint) {
-#pragma unroll
-                for (int q = 0; q < 8; ++q) sg[q] = p.signs[off + j + q];
-                if (p.awq) {
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) sc[q] = p.awq[off + j + q];
-                }
-            }
+        auto emit = [&](int j, const float (&sg)[8], const float (&sc)[8]) {
+            uint16_t op[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
                 float t = buf[fht_slot(j + q)];
@@ -92,8 +241,23 @@ __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
                     t = t * sg[q] * inv;
                     if (p.awq) t = t / sc[q];
                 }
-                store_any(p.out, row + off + j + q, p.dtype, t);
+                if (p.ap) {
+                    const int in_bf16 = p.dtype == FLUTE_BF16;
+                    uint16_t a = round_act(t, in_bf16);
+                    if (in_bf16 != p.ap_bf16) a = round_act(in_bf16 ? bf2f(a) : h2f(a), p.ap_bf16);
+                    op[q] = a;
+                } else {
+                    store_any(p.out, orow + off + j + q, p.dtype, t);
+                }
             }
+            if (p.ap) store_operand_order(p, blockIdx.x, off + j, op);
+        };
+        if (j0 < count) emit(j0, sg0, sc0);
+        if (j1 < count) emit(j1, sg1, sc1);
+        for (int j = j1 + kFhtThreads * 8; j < count; j += kFhtThreads * 8) {
+            float sg[8], sc[8];
+            load_mul(j, sg, sc);
+            emit(j, sg, sc);
         }
         __syncthreads();
         off += count;
@@ -104,28 +268,31 @@ __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
 
 }  // namespace flute
 
-using namespace flute;
+namespace flute {
 
-extern "C" flute_status flute_fht(const void *x, const float *signs, const float *awq, void *out,
-                                  int M, int K, int dtype, int adjoint, int block, void *stream) {
-    FLUTE_REQUIRE(x && out && signs, FLUTE_ERR_INVALID, "flute_fht: x, signs and out must not be NULL");
-    FLUTE_REQUIRE(dtype == FLUTE_F16 || dtype == FLUTE_BF16 || dtype == FLUTE_F32, FLUTE_ERR_INVALID,
-                  "flute_fht: dtype must be float16, bfloat16 or float32");
-    FLUTE_REQUIRE(M >= 0, FLUTE_ERR_INVALID, "flute_fht: M must be >= 0");
-    FLUTE_REQUIRE(K >= 32 && K % 32 == 0 && K <= 65504, FLUTE_ERR_INVALID,
-                  "flute_fht: K must be a multiple of 32 in [32, 65504] (got %d)", K);
-    FLUTE_REQUIRE(!(awq && adjoint), FLUTE_ERR_INVALID,
-                  "flute_fht: the awq-compensated transform exists in the forward direction only");
+flute_status fht_launch(const void *x, int64_t ldx, const float *signs, const float *awq, void *out,
+                        int64_t ldo, int M, int K, int dtype, int adjoint, int block,
+                        hipStream_t stream, const FhtOperandOut *operand) {
     FhtParams p;
     p.x = x;
     p.out = out;
     p.signs = signs;
     p.awq = awq;
+    p.ldx = ldx;
+    p.ldo = ldo;
     p.K = K;
     p.dtype = dtype;
     p.adjoint = adjoint ? 1 : 0;
     p.block = block;
     p.chunk = 0;
+    p.ap = operand ? operand->ap : nullptr;
+    p.ap_M = M;
+    p.ap_mblk_pad = operand ? operand->mblk_pad : 0;
+    p.ap_bf16 = operand ? operand->lut_bf16 : 0;
+    const bool io16 = dtype != FLUTE_F32;
+    p.vec_io = io16 && ((uintptr_t)x & 15) == 0 && ldx % 8 == 0 &&
+               (operand || (((uintptr_t)out & 15) == 0 && ldo % 8 == 0));
+    p.vec_mul = ((uintptr_t)signs & 15) == 0 && (!awq || ((uintptr_t)awq & 15) == 0);
     size_t lds_bytes;
     if (block > 0) {
         FLUTE_REQUIRE(is_pow2(block) && block >= 32 && block <= 16384 && K % block == 0,
@@ -141,14 +308,33 @@ extern "C" flute_status flute_fht(const void *x, const float *signs, const float
                       segs.len[0]);
         lds_bytes = (size_t)segs.len[0] * 4;
     }
-    if (M == 0) return FLUTE_OK;
+    const int rows = operand ? operand->mblk_pad * 16 : M;
+    if (rows == 0) return FLUTE_OK;
     static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
         FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)fht_kernel,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
         attr_done = true;
     }
-    hipLaunchKernelGGL(fht_kernel, dim3(M), dim3(kFhtThreads), lds_bytes, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(fht_kernel, dim3(rows), dim3(kFhtThreads), lds_bytes, stream, p);
     FLUTE_HIP_CHECK(hipGetLastError());
     return FLUTE_OK;
+}
+
+}  // namespace flute
+
+using namespace flute;
+
+extern "C" flute_status flute_fht(const void *x, const float *signs, const float *awq, void *out,
+                                  int M, int K, int dtype, int adjoint, int block, void *stream) {
+    FLUTE_REQUIRE(x && out && signs, FLUTE_ERR_INVALID, "flute_fht: x, signs and out must not be NULL");
+    FLUTE_REQUIRE(dtype == FLUTE_F16 || dtype == FLUTE_BF16 || dtype == FLUTE_F32, FLUTE_ERR_INVALID,
+                  "flute_fht: dtype must be float16, bfloat16 or float32");
+    FLUTE_REQUIRE(M >= 0, FLUTE_ERR_INVALID, "flute_fht: M must be >= 0");
+    FLUTE_REQUIRE(K >= 32 && K % 32 == 0 && K <= 65504, FLUTE_ERR_INVALID,
+                  "flute_fht: K must be a multiple of 32 in [32, 65504] (got %d)", K);
+    FLUTE_REQUIRE(!(awq && adjoint), FLUTE_ERR_INVALID,
+                  "flute_fht: the awq-compensated transform exists in the forward direction only");
+    return fht_launch(x, K, signs, awq, out, K, M, K, dtype, adjoint, block, (hipStream_t)stream,
+                      nullptr);
 }

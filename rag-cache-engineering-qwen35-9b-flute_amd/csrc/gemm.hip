@@ -235,17 +235,23 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     float *xb = base + p_floats;
     u4_t *Ap = (u4_t *)(xb + xb_floats);
     p.Ap = Ap;
-    if (w->signs) {
-        // rotated copy of the activations (the transform needs whole rows), then the
-        // ordinary pre-pass on it
-        void *Arot = (void *)(Ap + (size_t)p.G * 2 * p.mblk_pad * 64);
-        st = flute_fht(A, w->signs, w->awq, Arot, M, w->K, act_dtype, 0, w->rot_block, stream_);
+    if (w->signs && w->R == 0) {
+        // the rotation writes the operand image itself: one launch instead of two
+        FhtOperandOut image_out = {(uint32_t *)Ap, p.mblk_pad, (int)(w->lut_dtype == FLUTE_BF16)};
+        st = fht_launch(A, lda, w->signs, w->awq, nullptr, 0, M, w->K, act_dtype, 0, w->rot_block,
+                        stream, &image_out);
         if (st != FLUTE_OK) return st;
-        A = Arot;
-        lda = w->K;
-    }
-
-    {
+    } else {
+        if (w->signs) {
+            // the residual coefficients need the rotated rows as rows: rotated copy first,
+            // then the ordinary pre-pass on it
+            void *Arot = (void *)(Ap + (size_t)p.G * 2 * p.mblk_pad * 64);
+            st = fht_launch(A, lda, w->signs, w->awq, Arot, w->K, M, w->K, act_dtype, 0,
+                            w->rot_block, stream, nullptr);
+            if (st != FLUTE_OK) return st;
+            A = Arot;
+            lda = w->K;
+        }
         const int64_t total = (int64_t)p.G * 2 * p.mblk_pad * 64;
         const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
         hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,

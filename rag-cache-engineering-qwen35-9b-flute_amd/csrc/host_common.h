@@ -10,9 +10,6 @@ namespace flute {
 // mode: 0 = GEMV, 1 = GEMM / dequant.
 flute_status validate_linear(const flute_linear *w, int mode, const char *who);
 
-// K-split the GEMV launchers use for `tiles` 128-row workgroup columns over
-// G = K/64 tiles of K.
-
 // Split-K workspace of the current device: `floats` fp32 partial sums and
 // `ints` zero-initialised tickets.  Grows geometrically, never shrinks; the
 // tickets are zeroed once at allocation and every kernel leaves them at zero.
@@ -20,6 +17,18 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who);
 // (the same contract as upstream include/flute/gemv_host.h:31-38).
 flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float **P,
                            int **tickets);
+
+// The Walsh-Hadamard rotation of flute_fht with row strides, and optionally with its
+// output written in the operand order of the LUT GEMM (the image the GEMM's activation
+// pre-pass would produce from the rotated rows, padding rows zeroed) instead of as rows.
+struct FhtOperandOut {
+    uint32_t *ap;       // Ap[g][j][m / 16][lane][4 dwords]
+    int mblk_pad;       // 16-row blocks the image holds per half tile
+    int lut_bf16;       // 16-bit type of the image
+};
+flute_status fht_launch(const void *x, int64_t ldx, const float *signs, const float *awq, void *out,
+                        int64_t ldo, int M, int K, int dtype, int adjoint, int block,
+                        hipStream_t stream, const FhtOperandOut *operand);
 
 inline bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 inline int ilog2(int v) { return 31 - __builtin_clz((unsigned)v); }

@@ -57,6 +57,31 @@ def test_fht_block_mode_and_round_trip():
         fx._C.fht_forward(make_x(1, 100, dtype=torch.float32).to(DEV), torch.ones(100).to(DEV))
 
 
+@pytest.mark.parametrize("block", [32, 64, 128, 256, 512, 2048])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_fht_every_block_size_bit_exact(block, dtype):
+    """Blocks up to 256 columns are transformed in registers, larger ones in LDS: both
+    must give the reference butterfly's bits, forward and adjoint, also in place and on
+    rows that do not start on a 16-byte boundary."""
+    K, M = 6144, 5
+    signs = O.rotation_signs(K, block)
+    x = make_x(M, K, seed=block, dtype=dtype)
+    xd, sd = x.to(DEV), signs.to(DEV)
+    y = fx._C.fht_forward(xd, sd, block=block).cpu()
+    assert y.dtype == dtype and torch.equal(y, O.block_fht_reference(x, block, signs))
+    ya = fx._C.fht_backward(xd, sd, block=block).cpu()
+    xs = (x.float() * signs).to(torch.float32)
+    assert torch.equal(ya, O.block_fht_reference(xs, block).to(dtype))
+    z = xd.clone()
+    fx._C.fht_inplace_(z, sd, block=block)
+    assert torch.equal(z.cpu(), y)
+    # a view whose rows start 2 (or 4) bytes into a 16-byte line
+    off = torch.zeros(M * K + 1, dtype=dtype, device=DEV)
+    off[1:] = xd.reshape(-1)
+    yo = fx._C.fht_forward(off[1:].reshape(M, K), sd, block=block).cpu()
+    assert torch.equal(yo, y)
+
+
 @pytest.mark.parametrize("bits", [1, 2, 3, 4])
 @pytest.mark.parametrize("gs", [16, 128, 512])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -176,27 +176,47 @@ def test_module_kernel_mode_matches_reference_mode_prefill(M, spec, route, rot):
     assert list(pm.ROUTE_CENSUS) == [route]
 
 
-def test_gemm_with_rotation_through_the_c_abi():
-    """flute_gemm rotates its input itself when the descriptor carries signs
-    (block-128 form and the full-K form), M = 8 as in the rotated-input configuration."""
-    N, K, M = 512, 4096, 8
-    w = make_weight(N, K, seed=11, device=DEV)
-    x = make_x(M, K, seed=12, dtype=torch.bfloat16)
-    xd = x.to(DEV)
+@pytest.mark.parametrize("M,lda_pad,act,lut,rank", [
+    (8, 0, torch.bfloat16, torch.float16, 0),       # the rotated-input configuration
+    (8, 0, torch.float16, torch.float16, 0),
+    (40, 0, torch.bfloat16, torch.bfloat16, 0),     # several 16-row blocks, padded rows
+    (24, 64, torch.bfloat16, torch.float16, 0),     # rows of A further apart than K
+    (100, 0, torch.float16, torch.float16, 0),      # 64-row workgroups
+    (8, 0, torch.float16, torch.float16, 4),        # residual: rotated rows are kept as rows
+    (24, 64, torch.float16, torch.float16, 4),
+])
+def test_gemm_with_rotation_through_the_c_abi(M, lda_pad, act, lut, rank):
+    """flute_gemm rotates its input itself when the descriptor carries signs (block-128
+    form and the full-K form).  Without a residual the rotation writes the activations
+    straight in the order the matrix cores read them; with one, as rows first."""
+    N, K = 512, 4096
+    w = make_weight(N, K, seed=11, lut_dtype=lut, act_dtype=act, rank=rank, device=DEV)
+    x = make_x(M, K, seed=12, dtype=act)
+    lda = K + lda_pad
+    xd = torch.zeros(M, lda, dtype=act, device=DEV)
+    xd[:, :K] = x.to(DEV)
     for block in (128, 0):
         signs = O.rotation_signs(K, 3)
         sd = signs.to(DEV)
         d = _desc(w)
         d.signs, d.rot_block = sd.data_ptr(), block
-        C = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
-        st = _lib.lib.flute_gemm(ctypes.byref(d), xd.data_ptr(), C.data_ptr(), M, K, N, _lib.BF16,
+        if rank:
+            d.resA, d.resB, d.R = w["resA_d"].data_ptr(), w["resB_d"].data_ptr(), rank
+        C = torch.zeros(M, N, dtype=act, device=DEV)
+        st = _lib.lib.flute_gemm(ctypes.byref(d), xd.data_ptr(), C.data_ptr(), M, lda, N,
+                                 _lib.F16 if act == torch.float16 else _lib.BF16,
                                  torch.cuda.current_stream().cuda_stream)
         assert st == 0, _lib.last_error()
         xr = O.block_fht_reference(x, 128, signs) if block else O.fht_reference(x, signs)
-        # the rotated activations are rounded to bf16 before the GEMM, then cast to the
-        # LUT's fp16 (exact for these magnitudes)
-        ref = _exact(w, xr.to(torch.bfloat16).half()).to(torch.bfloat16)
-        assert rel_l2(C.cpu(), ref) <= 4e-3
+        # the rotated activations are rounded to the activation type before the GEMM, then
+        # cast to the LUT's type (exact for these magnitudes)
+        xr = xr.to(act)
+        ref = O.linear_exact(xr.to(lut), w["blob"].numpy(), w["lut"], N, K, w["gs"], w["bits"],
+                             None, None, 0, None, None, None).double()
+        if rank:
+            ref = ref + (xr.double() @ w["resB"].double().t()) @ w["resA"].double().t()
+        tol = 1.5e-3 if act == torch.float16 else 4e-3
+        assert rel_l2(C.cpu(), ref.to(act)) <= tol
 
 
 @pytest.mark.parametrize("rot", [False, True])
