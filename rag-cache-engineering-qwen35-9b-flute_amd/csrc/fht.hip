@@ -6,6 +6,7 @@
 #include <atomic>
 
 #include <cmath>
+#include <cstdlib>
 
 namespace flute {
 
@@ -70,104 +71,213 @@ __device__ __forceinline__ void load_mul8(const float *m, int k, int vec, float 
     }
 }
 
-// Equal blocks of at most 256 columns without the LDS buffer.  A thread holds eight
-// consecutive columns: the stages of length 1, 2, 4 are butterflies between its own
-// registers, the stages of length 8 ... block/2 pair it with the lane whose number differs
-// in one bit (ds_swizzle: the LDS crossbar, no memory access).  The lower lane of a pair
-// keeps a + b and the upper a - b, formed as fma(mine, +-1, other): the product is exact,
-// so every value sees the same single rounding per stage, in the same ascending order, as
-// in the buffered butterfly, and the result is bit-identical to it.  One memory round
-// trip, no barrier.  The lanes of a block are always in the same step of the loop
-// (a step covers 2048 columns, a multiple of every block), so a lane's partners are active.
+// Eight consecutive columns of a row as fp32, already multiplied by what the direction
+// applies before the butterfly (signs for the adjoint, the scale for the compensated
+// forward transform); sg/sc keep the multipliers the output needs.
+__device__ __forceinline__ void load_cols8(const FhtParams &p, int64_t row, int k, float (&f)[8],
+                                           float (&sg)[8], float (&sc)[8]) {
+    const int bf16 = p.dtype == FLUTE_BF16;
+    if (p.vec_io) {
+        const uint4 raw = *(const uint4 *)((const uint16_t *)p.x + row + k);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint16_t h = (uint16_t)(w[q >> 1] >> (16 * (q & 1)));
+            f[q] = bf16 ? bf2f(h) : h2f(h);
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) f[q] = load_any(p.x, row + k + q, p.dtype);
+    }
+    load_mul8(p.signs, k, p.vec_mul, sg);
+    if (p.awq) load_mul8(p.awq, k, p.vec_mul, sc);
+    if (p.adjoint || p.awq) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) f[q] *= p.adjoint ? sg[q] : sc[q];
+    }
+}
+
+// The transformed eight columns out: scaled, (forward) signed and de-scaled, one rounding
+// to the I/O type, as rows or in the GEMM's operand order.
+__device__ __forceinline__ void store_cols8(const FhtParams &p, int64_t orow, int k, float inv,
+                                            const float (&f)[8], const float (&sg)[8],
+                                            const float (&sc)[8]) {
+    const int bf16 = p.dtype == FLUTE_BF16;
+    uint16_t op[8];
+    float t[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        if (p.adjoint) {
+            t[q] = f[q] * inv;
+        } else {
+            t[q] = f[q] * sg[q] * inv;
+            if (p.awq) t[q] = t[q] / sc[q];
+        }
+        if (p.dtype != FLUTE_F32) {
+            uint16_t a = round_act(t[q], bf16);
+            if (p.ap && bf16 != p.ap_bf16) a = round_act(bf16 ? bf2f(a) : h2f(a), p.ap_bf16);
+            op[q] = a;
+        }
+    }
+    if (p.ap) {
+        store_operand_order(p, blockIdx.x, k, op);
+    } else if (p.dtype == FLUTE_F32) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ((float *)p.out)[orow + k + q] = t[q];
+    } else if (p.vec_io) {
+        *(uint4 *)((uint16_t *)p.out + orow + k) =
+            make_uint4((uint32_t)op[0] | ((uint32_t)op[1] << 16),
+                       (uint32_t)op[2] | ((uint32_t)op[3] << 16),
+                       (uint32_t)op[4] | ((uint32_t)op[5] << 16),
+                       (uint32_t)op[6] | ((uint32_t)op[7] << 16));
+    } else {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ((uint16_t *)p.out)[orow + k + q] = op[q];
+    }
+}
+
+// Stages of length 1, 2, 4 between a thread's own eight columns.
+__device__ __forceinline__ void stages_in_thread(float (&f)[8]) {
+#pragma unroll
+    for (int len = 1; len < 8; len <<= 1) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            if ((q & len) == 0) {
+                const float a = f[q], c = f[q | len];
+                f[q] = a + c;
+                f[q | len] = a - c;
+            }
+        }
+    }
+}
+
+// One stage against the lane whose number differs in bit M (M = 1 ... 16: ds_swizzle,
+// the LDS crossbar without a memory access).  The lower lane of a pair keeps a + b and
+// the upper a - b, formed as fma(mine, +-1, other): the product is exact, so every value
+// sees the same single rounding per stage as in the buffered butterfly.
+template <int M>
+__device__ __forceinline__ void stage_across_lanes(float (&f)[8], int lane) {
+    const float sgn = (lane & M) ? -1.0f : 1.0f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        const float other = __int_as_float(
+            __builtin_amdgcn_ds_swizzle(__float_as_int(f[q]), (M << 10) | 0x1f));
+        f[q] = fmaf(f[q], sgn, other);
+    }
+}
+
+// Equal blocks of at most 256 columns without the LDS buffer: three stages in a thread's
+// registers, the stages of length 8 ... block/2 across lanes, in the same ascending order
+// as the buffered butterfly and bit-identical to it.  One memory round trip, no barrier.
+// The lanes of a block are always in the same step of the loop (a step covers 2048
+// columns, a multiple of every block), so a lane's partners are active.
 __device__ __forceinline__ void fht_blocks_inwave(const FhtParams &p, int64_t row, int64_t orow,
                                                   int tid) {
     const int nst = 31 - __builtin_clz((unsigned)p.block);
     const float inv = inv_sqrt_pow2(nst);
     const int lane = tid & 63;
     const int pair_lanes = p.block >> 3;               // lanes of one block: 4 ... 32
-    const int bf16 = p.dtype == FLUTE_BF16;
+    // one step at a time: holding several steps of loads in registers measured slower
+    // (K = 4096: 5.4 us against 3.8 us per launch)
     for (int j = tid * 8; j < p.K; j += kFhtThreads * 8) {
         float f[8], sg[8], sc[8];
-        if (p.vec_io) {
-            const uint4 raw = *(const uint4 *)((const uint16_t *)p.x + row + j);
-            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                const uint16_t h = (uint16_t)(w[q >> 1] >> (16 * (q & 1)));
-                f[q] = bf16 ? bf2f(h) : h2f(h);
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) f[q] = load_any(p.x, row + j + q, p.dtype);
-        }
-        load_mul8(p.signs, j, p.vec_mul, sg);
-        if (p.awq) load_mul8(p.awq, j, p.vec_mul, sc);
-        if (p.adjoint || p.awq) {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) f[q] *= p.adjoint ? sg[q] : sc[q];
-        }
-#pragma unroll
-        for (int len = 1; len < 8; len <<= 1) {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                if ((q & len) == 0) {
-                    const float a = f[q], c = f[q | len];
-                    f[q] = a + c;
-                    f[q | len] = a - c;
-                }
-            }
-        }
-        // and_mask 0x1f, or_mask 0, xor_mask m: lane ^ m inside each half of the wavefront
-#define FLUTE_XOR_STAGE(m)                                                                   \
-        if (pair_lanes > (m)) {                                                              \
-            const float sgn = (lane & (m)) ? -1.0f : 1.0f;                                   \
-            _Pragma("unroll") for (int q = 0; q < 8; ++q) {                                  \
-                const float other = __int_as_float(__builtin_amdgcn_ds_swizzle(              \
-                    __float_as_int(f[q]), ((m) << 10) | 0x1f));                              \
-                f[q] = fmaf(f[q], sgn, other);                                               \
-            }                                                                                \
-        }
-        FLUTE_XOR_STAGE(1)
-        FLUTE_XOR_STAGE(2)
-        FLUTE_XOR_STAGE(4)
-        FLUTE_XOR_STAGE(8)
-        FLUTE_XOR_STAGE(16)
-#undef FLUTE_XOR_STAGE
-        uint16_t op[8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            float t;
-            if (p.adjoint) {
-                t = f[q] * inv;
-            } else {
-                t = f[q] * sg[q] * inv;
-                if (p.awq) t = t / sc[q];
-            }
-            f[q] = t;
-            if (p.dtype != FLUTE_F32) {
-                uint16_t a = round_act(t, bf16);
-                if (p.ap && bf16 != p.ap_bf16) a = round_act(bf16 ? bf2f(a) : h2f(a), p.ap_bf16);
-                op[q] = a;
-            }
-        }
-        if (p.ap) {
-            store_operand_order(p, blockIdx.x, j, op);
-        } else if (p.dtype == FLUTE_F32) {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) ((float *)p.out)[orow + j + q] = f[q];
-        } else if (p.vec_io) {
-            *(uint4 *)((uint16_t *)p.out + orow + j) =
-                make_uint4((uint32_t)op[0] | ((uint32_t)op[1] << 16),
-                           (uint32_t)op[2] | ((uint32_t)op[3] << 16),
-                           (uint32_t)op[4] | ((uint32_t)op[5] << 16),
-                           (uint32_t)op[6] | ((uint32_t)op[7] << 16));
-        } else {
-#pragma unroll
-            for (int q = 0; q < 8; ++q) ((uint16_t *)p.out)[orow + j + q] = op[q];
-        }
+        load_cols8(p, row, j, f, sg, sc);
+        stages_in_thread(f);
+        if (pair_lanes > 1) stage_across_lanes<1>(f, lane);
+        if (pair_lanes > 2) stage_across_lanes<2>(f, lane);
+        if (pair_lanes > 4) stage_across_lanes<4>(f, lane);
+        if (pair_lanes > 8) stage_across_lanes<8>(f, lane);
+        if (pair_lanes > 16) stage_across_lanes<16>(f, lane);
+        store_cols8(p, orow, j, inv, f, sg, sc);
     }
 }
 
+// One power-of-two segment of 512 ... 8192 columns starting at column `off`.  The first
+// nine stages (lengths 1 ... 256) run as in fht_blocks_inwave, the last of them against
+// the lane 32 away (ds_bpermute); the remaining stages (lengths 512 ... b/2, at most
+// four) are one pass over the fp32 buffer in LDS.  Same butterflies in the same ascending
+// order as fht_lds alone, so bit-identical; one memory round trip instead of two, two
+// barriers instead of five, a third of the LDS traffic.  A thread holds up to S steps of
+// eight columns; b/8 is a multiple of 64, so wavefronts are active as a whole, and a
+// step a thread does not have repeats its first one (loads stay unconditional).
+template <int S>
+__device__ __forceinline__ void fht_segment_fast(const FhtParams &p, int64_t row, int64_t orow,
+                                                 int off, int b, int nst, float *buf, int tid) {
+    const float inv = inv_sqrt_pow2(nst);
+    const int lane = tid & 63;
+    const int j0 = tid * 8;
+    constexpr int STEP = kFhtThreads * 8;
+    const bool one = j0 < b;
+    float f[S][8], sg[S][8], sc[S][8];
+    if (one) {
+#pragma unroll
+        for (int h = 0; h < S; ++h)
+            load_cols8(p, row, off + (j0 + h * STEP < b ? j0 + h * STEP : j0), f[h], sg[h], sc[h]);
+#pragma unroll
+        for (int h = 0; h < S; ++h) stages_in_thread(f[h]);
+#pragma unroll
+        for (int h = 0; h < S; ++h) stage_across_lanes<1>(f[h], lane);
+#pragma unroll
+        for (int h = 0; h < S; ++h) stage_across_lanes<2>(f[h], lane);
+#pragma unroll
+        for (int h = 0; h < S; ++h) stage_across_lanes<4>(f[h], lane);
+#pragma unroll
+        for (int h = 0; h < S; ++h) stage_across_lanes<8>(f[h], lane);
+#pragma unroll
+        for (int h = 0; h < S; ++h) stage_across_lanes<16>(f[h], lane);
+        const float sgn = (lane & 32) ? -1.0f : 1.0f;
+        const int partner = (lane ^ 32) << 2;
+#pragma unroll
+        for (int h = 0; h < S; ++h)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const float other = __int_as_float(
+                    __builtin_amdgcn_ds_bpermute(partner, __float_as_int(f[h][q])));
+                f[h][q] = fmaf(f[h][q], sgn, other);
+            }
+    }
+    if (nst > 9) {                                     // uniform: stages of length 512 and up
+        if (one) {
+#pragma unroll
+            for (int h = 0; h < S; ++h) {
+                if (j0 + h * STEP < b) {
+                    const int s0 = fht_slot(j0 + h * STEP);   // multiple of 8: slot(j + q) = s0 ^ q
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) buf[s0 ^ q] = f[h][q];
+                }
+            }
+        }
+        __syncthreads();
+        switch (nst - 9) {
+            case 1: fht_pass<1>(buf, b, 9, tid, kFhtThreads); break;
+            case 2: fht_pass<2>(buf, b, 9, tid, kFhtThreads); break;
+            case 3: fht_pass<3>(buf, b, 9, tid, kFhtThreads); break;
+            default: fht_pass<4>(buf, b, 9, tid, kFhtThreads); break;
+        }
+        __syncthreads();
+        if (one) {
+#pragma unroll
+            for (int h = 0; h < S; ++h) {
+                if (j0 + h * STEP < b) {
+                    const int s0 = fht_slot(j0 + h * STEP);
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) f[h][q] = buf[s0 ^ q];
+                }
+            }
+        }
+        __syncthreads();                               // the next segment reuses the buffer
+    }
+    if (one) {
+#pragma unroll
+        for (int h = 0; h < S; ++h)
+            if (j0 + h * STEP < b) store_cols8(p, orow, off + j0 + h * STEP, inv, f[h], sg[h], sc[h]);
+    }
+}
+
+// MAXS: steps of eight columns a thread may hold in the register-resident segment path
+// (0: every segment through the LDS buffer; 2: segments up to 4096 columns in registers;
+// 4: up to 8192, at twice the registers).
+template <int MAXS>
 __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     float *buf = (float *)lds;
@@ -194,6 +304,16 @@ __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
         } else {
             nstages = 31 - __builtin_clz((unsigned)(p.K - off));
             count = 1 << nstages;
+        }
+        if constexpr (MAXS > 0) {
+            if (p.block == 0 && count >= 512 && count <= kFhtThreads * 8 * MAXS) {
+                if (MAXS == 2 || count <= kFhtThreads * 16)
+                    fht_segment_fast<2>(p, row, orow, off, count, nstages, buf, tid);
+                else
+                    fht_segment_fast<MAXS>(p, row, orow, off, count, nstages, buf, tid);
+                off += count;
+                continue;
+            }
         }
         const float inv = inv_sqrt_pow2(nstages);
         // The output multipliers of a thread's first two steps are requested together
@@ -294,6 +414,7 @@ flute_status fht_launch(const void *x, int64_t ldx, const float *signs, const fl
                (operand || (((uintptr_t)out & 15) == 0 && ldo % 8 == 0));
     p.vec_mul = ((uintptr_t)signs & 15) == 0 && (!awq || ((uintptr_t)awq & 15) == 0);
     size_t lds_bytes;
+    bool wide = false;
     if (block > 0) {
         FLUTE_REQUIRE(is_pow2(block) && block >= 32 && block <= 16384 && K % block == 0,
                       FLUTE_ERR_INVALID,
@@ -307,16 +428,36 @@ flute_status fht_launch(const void *x, int64_t ldx, const float *signs, const fl
                       "flute_fht: segment of %d columns exceeds the 16384-column LDS tile",
                       segs.len[0]);
         lds_bytes = (size_t)segs.len[0] * 4;
+        wide = segs.len[0] > kFhtThreads * 16 && segs.len[0] <= kFhtThreads * 32;
     }
     const int rows = operand ? operand->mblk_pad * 16 : M;
     if (rows == 0) return FLUTE_OK;
     static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)fht_kernel,
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)fht_kernel<2>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)fht_kernel<0>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)fht_kernel<4>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
         attr_done = true;
     }
-    hipLaunchKernelGGL(fht_kernel, dim3(rows), dim3(kFhtThreads), lds_bytes, stream, p);
+    // Which variant: the register-resident segment path wins wherever it applies, except
+    // that its wide form (segments of 8192 columns, 270 registers, one workgroup per CU)
+    // loses to the buffered kernel once there are many rows (K = 12288: 12.4 us against
+    // 21.0 us for one row, 52.6 us against 40.3 us for 1024 rows).  FLUTE_FHT_STEPS = 0, 2
+    // or 4 forces a variant (tuning and test knob).
+    int steps = wide ? (rows <= 512 ? 4 : 0) : 2;
+    if (const char *e = getenv("FLUTE_FHT_STEPS")) {
+        const int v = atoi(e);
+        if (v == 0 || v == 2 || v == 4) steps = v;
+    }
+    if (steps == 0)
+        hipLaunchKernelGGL(fht_kernel<0>, dim3(rows), dim3(kFhtThreads), lds_bytes, stream, p);
+    else if (steps == 4)
+        hipLaunchKernelGGL(fht_kernel<4>, dim3(rows), dim3(kFhtThreads), lds_bytes, stream, p);
+    else
+        hipLaunchKernelGGL(fht_kernel<2>, dim3(rows), dim3(kFhtThreads), lds_bytes, stream, p);
     FLUTE_HIP_CHECK(hipGetLastError());
     return FLUTE_OK;
 }

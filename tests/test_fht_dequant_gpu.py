@@ -57,6 +57,22 @@ def test_fht_block_mode_and_round_trip():
         fx._C.fht_forward(make_x(1, 100, dtype=torch.float32).to(DEV), torch.ones(100).to(DEV))
 
 
+@pytest.mark.parametrize("steps", ["0", "2", "4"])
+@pytest.mark.parametrize("K", [1536, 4096, 12288, 24576])
+def test_fht_every_kernel_variant_bit_exact(monkeypatch, steps, K):
+    """Segments are transformed through the LDS buffer, or up to 4096 / 8192 columns in
+    registers with one LDS pass; the library picks by K and the number of rows.  Each
+    variant forced in turn (FLUTE_FHT_STEPS, read per call) must give the reference's bits."""
+    monkeypatch.setenv("FLUTE_FHT_STEPS", steps)
+    signs = O.rotation_signs(K, 7)
+    for dtype in (torch.float32, torch.bfloat16):
+        x = make_x(3, K, seed=K, dtype=dtype)
+        y = fht.fht_apply(x.to(DEV), signs.to(DEV), backend="kernel").cpu()
+        assert torch.equal(y, O.fht_reference(x, signs))
+        ya = fht.fht_adjoint(x.to(DEV), signs.to(DEV), backend="kernel").cpu()
+        assert torch.equal(ya, O.fht_adjoint_reference(x, signs))
+
+
 @pytest.mark.parametrize("block", [32, 64, 128, 256, 512, 2048])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_fht_every_block_size_bit_exact(block, dtype):
