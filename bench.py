@@ -230,8 +230,47 @@ def _gemm_section(torch, _lib, ctypes, sets, gen, dev, O):
         tf = 2.0 * M * I * H / us / 1e6
         res[M] = {"us_per_call": round(us, 2), "tflops": round(tf, 1),
                   "frac_mfma": round(tf / MFMA_PEAK_TFLOPS, 4), "parity_rel_l2": err}
+    # the rotated-input configuration at M = 8: block-128 Hadamard rotation of the rows in
+    # front of the same GEMM (one rotation launch that writes the operand order + the kernel)
+    M = 8
+    signs = (torch.randint(0, 2, (H,), device=dev, generator=gen).float() * 2 - 1).contiguous()
+    rot = []
+    for d in descs:
+        r = _lib.FluteLinear()
+        ctypes.memmove(ctypes.byref(r), ctypes.byref(d), ctypes.sizeof(r))
+        r.signs, r.rot_block = signs.data_ptr(), 128
+        rot.append(r)
+    A = torch.randn(M, H, device=dev, generator=gen).to(torch.bfloat16)
+    C = torch.empty(M, I, dtype=torch.bfloat16, device=dev)
+
+    def call_rot(i):
+        st = _lib.lib.flute_gemm(ctypes.byref(rot[i % len(rot)]), A.data_ptr(), C.data_ptr(),
+                                 M, H, I, _lib.BF16, torch.cuda.current_stream().cuda_stream)
+        if st != 0:
+            raise RuntimeError(_lib.last_error())
+
+    call_rot(0)
+    torch.cuda.synchronize()
+    blob, lut = sets[0]["t"][0][0], lut_bf[0]
+    per = (H // 64) * 4096
+    Ar = O.block_fht_reference(A.cpu(), 128, signs.cpu()).to(torch.bfloat16).double()
+    num = den = 0.0
+    for tile in (0, 41, 95):
+        Wt = O.dequant(blob[tile * per:(tile + 1) * per].cpu().numpy(), lut[tile:tile + 1].cpu(),
+                       128, H, GS, 4).double()
+        ref = Ar @ Wt.t()
+        got = C[:, tile * 128:(tile + 1) * 128].cpu().double()
+        num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
+    err = (num / den) ** 0.5
+    if err > 4e-3:
+        raise SystemExit(f"bench.py: rotated GEMM parity gate failed ({err:.2e})")
+    n = 48
+    us = _time_graph(torch, lambda: [call_rot(i) for i in range(n)]) / n * 1e3
+    rotated = {"us_per_call": round(us, 2), "parity_rel_l2": err,
+               "workload": "M=8, block-128 Hadamard rotation of the input + LUT-GEMM 4096->12288"}
     head = res[256]
-    return {"workload": "LUT-GEMM M=256: 4096->12288, idx4, group 128, bf16 LUT, bf16 activations, "
+    return {"rotated_input_M8": rotated,
+            "workload": "LUT-GEMM M=256: 4096->12288, idx4, group 128, bf16 LUT, bf16 activations, "
                         "bf16 MFMA fp32 accumulate; whole flute_gemm call (activation pre-pass + kernel)",
             "value": head["tflops"], "unit": "TFLOP/s", "peak": MFMA_PEAK_TFLOPS,
             "frac": head["frac_mfma"], "us_per_call": head["us_per_call"],
