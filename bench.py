@@ -167,6 +167,12 @@ def _gemv_section(torch, _lib, ctypes, sets, gen, dev, O):
         d.signs, d.rot_block = signs.data_ptr(), 128
         rot.append(d)
     run("gemv_4096x12288_fht128_fused", rot, I, H, x, keep, signs=signs, block=128)
+    # the widest weight of the model family: lm_head 4096 -> 248320 (0.5 GB of indices, upstream
+    # quotes its plain streamer on this shape); two weights in rotation are 1 GB
+    NV = 248320
+    ws = [_weights(torch, NV, H, gen, dev, torch.float16) for _ in range(2)]
+    run("gemv_lm_head_4096x248320", [_desc(_lib, b, l, NV, H) for b, l in ws], NV, H, x, ws)
+    del ws
     # narrow outputs: the library's own choice (it does not split K on this device) and the
     # forced K splits of the configuration beside it; enough weights to stay out of the caches
     for N in (1024, 512):
