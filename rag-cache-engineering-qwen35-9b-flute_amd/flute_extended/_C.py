@@ -43,8 +43,34 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None or t.numel() == 0 else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_of(t: torch.Tensor) -> int:
+    """Handle of torch's current stream on t's device (the raw query where this torch has
+    it: it skips building a Stream object on every call)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None
+                           else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _on_device_of:
+    """Device guard for a launch: a no-op when t's device is already current."""
+
+    def __init__(self, t: torch.Tensor):
+        idx = t.device.index
+        self._guard = None if idx is None or idx == torch.cuda.current_device() \
+            else torch.cuda.device(t.device)
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            self._guard.__exit__(*exc)
+        return False
 
 
 def _aligned16(t: torch.Tensor) -> torch.Tensor:
@@ -205,7 +231,7 @@ def _gemv(who, A, indices, lut, bitwidth, indices2, lut2, bitwidth2, resB, resA,
                            resB, resA, bias, group_size, signs, s, rot_block, gs_allowed,
                            max_rank)
     A = _aligned16(A)
-    with torch.cuda.device(A.device):
+    with _on_device_of(A):
         C = torch.empty((1, N), dtype=A.dtype, device=A.device)
         check(lib.flute_gemv(ctypes.byref(w), A.data_ptr(), C.data_ptr(), _ACT[A.dtype],
                              int(split), _stream_of(A)))
@@ -319,7 +345,7 @@ def qgemm_gemv_multi(A, seg_table, lut_dtype: Optional[torch.dtype] = None, spli
             _fail(f"{who}: segment {i} has no output pointer")
     arr = (ctypes.c_void_p * len(outs))(*outs)
     A = _aligned16(A)
-    with torch.cuda.device(A.device):
+    with _on_device_of(A):
         check(lib.flute_gemv_multi(descs, len(outs), A.data_ptr(), arr, _ACT[A.dtype],
                                    int(split), _stream_of(A)))
     return None
@@ -339,7 +365,7 @@ def qgemm_gemv_mlp(A, seg_table, C, lut_dtype: Optional[torch.dtype] = None, spl
         _fail(f"{who}: A and C must be CUDA (HIP) tensors")
     descs, _ = _seg_descs(who, A, seg_table, _ACT[lut_dtype or torch.float16])
     A = _aligned16(A)
-    with torch.cuda.device(A.device):
+    with _on_device_of(A):
         check(lib.flute_gemv_mlp(ctypes.byref(descs[0]), ctypes.byref(descs[1]), A.data_ptr(),
                                  C.data_ptr(), _ACT[A.dtype], int(split), _stream_of(A)))
     return C
@@ -358,7 +384,7 @@ def _gemm(who, A, indices, lut, bitwidth, indices2, lut2, bitwidth2, resB, resA,
     w, N, keep = _describe(who, A, K, indices, lut, bitwidth, indices2, lut2, bitwidth2,
                            resB, resA, bias, group_size, None, None, 0, gs_allowed, max_rank)
     A = _aligned16(A)
-    with torch.cuda.device(A.device):
+    with _on_device_of(A):
         C = torch.empty((M, N), dtype=A.dtype, device=A.device)
         check(lib.flute_gemm(ctypes.byref(w), A.data_ptr(), C.data_ptr(), M, K, N,
                              _ACT[A.dtype], _stream_of(A)))
@@ -424,7 +450,7 @@ def dequant_idxn(indices, lut, N: int, K: int, bitwidth: int, group_size: int):
                             group_size)
     if N2 != int(N):
         _fail(f"{who}: blob holds N={N2}, not {N}")
-    with torch.cuda.device(A.device):
+    with _on_device_of(A):
         W = torch.empty((N2, int(K)), dtype=lut.dtype, device=lut.device)
         check(lib.flute_dequant(ctypes.byref(w), 1, W.data_ptr(), _stream_of(A)))
     del keep
@@ -453,7 +479,7 @@ def _fht(who, x, signs, awq, out, adjoint, block=0):
         _fail(f"{who}: x must be contiguous")
     if not (x.is_cuda and signs.is_cuda and (awq is None or awq.is_cuda)):
         _fail(f"{who}: all tensors must be CUDA (HIP) tensors")
-    with torch.cuda.device(x.device):
+    with _on_device_of(x):
         if out is None:
             out = torch.empty_like(x)
         check(lib.flute_fht(x.data_ptr(), signs.data_ptr(), _ptr(awq), out.data_ptr(), M, K,
@@ -532,7 +558,7 @@ def embedding_gather(ids, indices, lut, N: int, K: int, bitwidth: int, group_siz
     flat = ids.reshape(-1).long().contiguous()
     if flat.numel() and (int(flat.min()) < 0 or int(flat.max()) >= N2):
         _fail(f"{who}: ids must lie in [0, {N2}) (got min {int(flat.min())}, max {int(flat.max())})")
-    with torch.cuda.device(A.device):
+    with _on_device_of(A):
         out = torch.empty((flat.numel(), int(K)), dtype=lut.dtype, device=lut.device)
         check(lib.flute_embedding(ctypes.byref(w), flat.data_ptr(), flat.numel(), out.data_ptr(),
                                   _stream_of(A)))

@@ -29,6 +29,8 @@ from __future__ import annotations
 
 from typing import Literal, Optional
 
+import functools
+
 import torch
 
 from . import _C
@@ -56,12 +58,25 @@ _LAYOUT_BITS = {"idx1": 1, "idx2": 2, "idx3": 3, "idx4": 4}
 LDS_BYTES_PER_CU = 160 * 1024
 
 
+_EMPTY = {}
+
+
+def _empty(device, dtype):
+    """One zero-element tensor per (device, dtype): the placeholders carry no data, so
+    every call can share them instead of allocating three new ones."""
+    key = (device, dtype)
+    t = _EMPTY.get(key)
+    if t is None:
+        t = _EMPTY[key] = torch.empty(0, dtype=dtype, device=device)
+    return t
+
+
 def _none_to_empty(A: torch.Tensor, indices2, lut2, resB, resA, bias, lut_dtype=None):
     """The `_C` convention: an absent operand is an empty tensor
     (upstream __init__.py:321-334)."""
-    e8 = torch.empty(0, dtype=torch.uint8, device=A.device)
-    e16 = torch.empty(0, dtype=A.dtype, device=A.device)
-    el = torch.empty(0, dtype=lut_dtype or A.dtype, device=A.device)
+    e8 = _empty(A.device, torch.uint8)
+    e16 = _empty(A.device, A.dtype)
+    el = _empty(A.device, lut_dtype or A.dtype)
     return (indices2 if indices2 is not None else e8,
             lut2 if lut2 is not None else el,
             resB if resB is not None else e16,
@@ -147,8 +162,14 @@ def gemv_stream_available() -> bool:
     return True
 
 
+@functools.lru_cache(maxsize=4096)
+def _lds_need(N: int, K: int, b1: int, b2: int, gs: int, fht: bool, rank: int) -> int:
+    return _C.gemv_lds_bytes(N, K, b1, b2, gs, fht=fht, residual_rank=rank)
+
+
 def _lds_ok(N, K, b1, b2, gs, fht, rank=0) -> bool:
-    need = _C.gemv_lds_bytes(N, K, b1, b2, gs, fht=fht, residual_rank=rank)
+    # pure host arithmetic of the shape: asked once per shape, not once per call
+    need = _lds_need(int(N), int(K), int(b1), int(b2), int(gs), bool(fht), int(rank))
     return 0 < need <= LDS_BYTES_PER_CU
 
 
