@@ -47,16 +47,16 @@ GemmShape choose_gemm_shape(int M, int tiles, int64_t index_bytes) {
     return {4, 4, 2, 1};
 }
 
-template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false>
+template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false, bool DIRECT = false>
 flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
     static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1, PERM>,
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1, PERM, DIRECT>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
                                             (int)kLdsPerCU));
         attr_done = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<MB, KW, MW, BF16, B1, PERM>), grid, dim3(64 * KW * MW), lds,
+    hipLaunchKernelGGL((gemm_kernel<MB, KW, MW, BF16, B1, PERM, DIRECT>), grid, dim3(64 * KW * MW), lds,
                        stream, p);
     FLUTE_HIP_CHECK(hipGetLastError());
     return FLUTE_OK;
@@ -68,6 +68,7 @@ template <bool BF16>
 flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 grid, int lds,
                                hipStream_t stream) {
     if (!BF16 && p.nstreams == 1 && p.bits[0] == 4 && p.rep_log2[0] == 6) {
+        if (s.mb == 1 && p.A8) return launch_gemm<1, 8, 1, false, 4, true, true>(p, grid, lds, stream);
         if (s.mb == 1) return launch_gemm<1, 8, 1, false, 4, true>(p, grid, lds, stream);
         if (s.mb == 2) return launch_gemm<2, 8, 1, false, 4, true>(p, grid, lds, stream);
         if (s.mw == 1) return launch_gemm<4, 8, 1, false, 4, true>(p, grid, lds, stream);
@@ -82,6 +83,10 @@ flute_status launch_gemm_bits(const GemmParams &p, dim3 grid, int lds, hipStream
     if (p.nstreams == 1) {
         switch (p.bits[0]) {
             case 4:
+                if constexpr (MB == 1) {
+                    if (p.rep_log2[0] == 6 && p.A8)
+                        return launch_gemm<MB, KW, MW, BF16, 4, true, true>(p, grid, lds, stream);
+                }
                 if (p.rep_log2[0] == 6) return launch_gemm<MB, KW, MW, BF16, 4, true>(p, grid, lds, stream);
                 return launch_gemm<MB, KW, MW, BF16, 4>(p, grid, lds, stream);
             case 3: return launch_gemm<MB, KW, MW, BF16, 3>(p, grid, lds, stream);
@@ -235,7 +240,23 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     float *xb = base + p_floats;
     u4_t *Ap = (u4_t *)(xb + xb_floats);
     p.Ap = Ap;
-    if (w->signs && w->R == 0) {
+    // One block of rows per wavefront on the single-stream 4-bit fast path: the kernel reads
+    // A itself (16-byte pieces of a row, put into operand order in registers), so the
+    // pre-pass launch is dropped.  Needs 16-byte aligned rows.
+    {
+        const int ngrp = w->group_size >= 128 ? 1 : 128 / w->group_size;
+        const bool fast = p.nstreams == 1 && w->b1 == 4 && ngrp <= 2 &&
+                          getenv("FLUTE_GEMM_NO_PERM") == nullptr;
+        if (shape.mb == 1 && fast && !w->signs && ((uintptr_t)A & 15) == 0 && lda % 8 == 0 &&
+            getenv("FLUTE_GEMM_NO_DIRECT") == nullptr) {
+            p.A8 = (const u4_t *)A;
+            p.lda8 = lda / 8;
+            p.a_bf16 = act_dtype == FLUTE_BF16;
+        }
+    }
+    if (p.A8) {
+        // nothing to prepare
+    } else if (w->signs && w->R == 0) {
         // the rotation writes the operand image itself: one launch instead of two
         FhtOperandOut image_out = {(uint32_t *)Ap, p.mblk_pad, (int)(w->lut_dtype == FLUTE_BF16)};
         st = fht_launch(A, lda, w->signs, w->awq, nullptr, 0, M, w->K, act_dtype, 0, w->rot_block,

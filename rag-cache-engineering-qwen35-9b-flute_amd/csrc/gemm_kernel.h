@@ -59,6 +59,9 @@ struct GemmParams {
                            // ztotal (several launches, one per stream, may share a fold)
     int out_bf16;          // dtype of C, resA, bias
     int vec_store;         // C rows allow 16-byte stores
+    const u4_t *A8;        // direct mode: A itself, rows of lda8 16-byte pieces, no pre-pass
+    int64_t lda8;
+    int a_bf16;            // dtype of A in direct mode
 #ifdef FLUTE_GEMM_TRACE
     unsigned long long *trace;   // [workgroup][16] timestamps, development builds only
 #endif
@@ -246,10 +249,37 @@ __device__ __forceinline__ void half_mma(const uint32_t (&Q)[4 * B], int j, cons
     }
 }
 
+// Direct mode of the one-block fast path: a lane has loaded eight consecutive k of its row
+// (piece c = lane >> 4 of the 32-k half tile), the matrix cores want the pairs
+// (2*kg, 2*kg + 1) of all four pieces.  With the four lanes that share a row (16 apart)
+// this is a 4 x 4 transpose of dwords: in round r every lane offers dword (kg + r) & 3 and
+// reads the offer of piece (kg - r) & 3, which is that piece's dword kg.
+__device__ __forceinline__ u4_t quad_transpose(u4_t v, int lane) {
+    const int kg = lane >> 4;
+    u4_t out = v;                                      // round 0: own piece, dword kg stays
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+        const int give = (kg + r) & 3, take = (kg - r) & 3;
+        const uint32_t offer = (give & 2) ? ((give & 1) ? v[3] : v[2]) : ((give & 1) ? v[1] : v[0]);
+        const uint32_t got = (uint32_t)__builtin_amdgcn_ds_bpermute(
+            (take * 16 + (lane & 15)) << 2, (int)offer);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) out[q] = (take == q) ? got : out[q];
+    }
+    // out[q] for q != kg now holds piece q's dword kg; the own piece contributes v[kg] at q = kg
+    const uint32_t own = (kg & 2) ? ((kg & 1) ? v[3] : v[2]) : ((kg & 1) ? v[1] : v[0]);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) out[q] = (kg == q) ? own : out[q];
+    return out;
+}
+
 // B1 > 0: single stream of that width.  B1 == 0: widths read from the
 // parameters, one or two streams.
-template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false>
+// DIRECT (one block per wavefront on the fast path only): the activations are read from A
+// itself and put into operand order in registers; no pre-pass launch.
+template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false, bool DIRECT = false>
 __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) {
+    static_assert(!DIRECT || (PERM && MB == 1), "direct activations: one block, fast path");
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int NT = 64 * KW * MW;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -266,13 +296,33 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     const bool active = mb0 < p.mblk_total;            // whole wavefront
     const int g0 = gbeg + kw;
     int left = (active && g0 < gend) ? (gend - g0 + KW - 1) / KW : 0;   // tiles of this wavefront
-    const int64_t jstep = (int64_t)p.mblk_pad * 64;    // u4 units between the halves of a tile
+    // u4 units between the halves of a tile (direct mode: 32 k of a row are four pieces)
+    const int64_t jstep = DIRECT ? 4 : (int64_t)p.mblk_pad * 64;
     // Ap is padded to whole workgroups of blocks (zeros), so every block index below
     // gridDim.y * MW * MB is loadable.
     // A wavefront without tiles addresses the first tile of the K range instead: its
     // loads below are then unconditional like everyone's, and the compiler can count them.
     const int g_first = left > 0 ? g0 : gbeg;
-    const u4_t *ap = p.Ap + ((int64_t)g_first * 2 * p.mblk_pad + mb0) * 64 + lane;
+    const int a_row = mb0 * 16 + rho;                  // direct mode: this lane's row of A
+    const bool a_row_valid = a_row < p.M;
+    const u4_t *ap = DIRECT
+        ? p.A8 + (int64_t)(a_row_valid ? a_row : 0) * p.lda8 + (int64_t)g_first * 8 + kg
+        : p.Ap + ((int64_t)g_first * 2 * p.mblk_pad + mb0) * 64 + lane;
+    // direct mode: raw piece -> operand (rows beyond M are zero; the activations are
+    // presented in the LUT's 16-bit type)
+    auto operand_of = [&](u4_t raw) -> u4_t {
+        if (!a_row_valid) raw = u4_t{0u, 0u, 0u, 0u};
+        if (p.a_bf16 != (int)BF16) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint16_t lo16 = (uint16_t)(raw[q] & 0xffffu), hi16 = (uint16_t)(raw[q] >> 16);
+                const float flo = p.a_bf16 ? bf2f(lo16) : h2f(lo16);
+                const float fhi = p.a_bf16 ? bf2f(hi16) : h2f(hi16);
+                raw[q] = (uint32_t)round_act(flo, BF16) | ((uint32_t)round_act(fhi, BF16) << 16);
+            }
+        }
+        return quad_transpose(raw, lane);
+    };
     auto load_a = [&](u4_t (&Aj)[MB], const u4_t *src) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) Aj[mb] = src[mb * 64];
@@ -383,7 +433,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 
             uint32_t Q[16];
             constexpr int64_t qstep = (int64_t)KW * 4096;
-            const int64_t astep = (int64_t)KW * 2 * p.mblk_pad * 64;
+            const int64_t astep = DIRECT ? (int64_t)KW * 8 : (int64_t)KW * 2 * p.mblk_pad * 64;
             auto stage_write = [&]() {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
@@ -408,7 +458,12 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             while (left > 0) {
                 stage_read();                             // this tile's chunk
                 __builtin_amdgcn_sched_barrier(0);
-                half_mma<4, MB, BF16, true>(Q, 0, A0, acc, lb, 8);
+                if constexpr (DIRECT) {
+                    const u4_t T0[1] = {operand_of(A0[0])};
+                    half_mma<4, MB, BF16, true>(Q, 0, T0, acc, lb, 8);
+                } else {
+                    half_mma<4, MB, BF16, true>(Q, 0, A0, acc, lb, 8);
+                }
                 if (left > 1) ap += astep;
                 load_a(A0, ap);                           // half a tile ahead of its use
                 // issue order activations -> tile: the wait for these activations at the
@@ -418,7 +473,12 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 if (left > 2) tp += qstep;
                 load_tile();                              // the tile after it
                 __builtin_amdgcn_sched_barrier(0);
-                half_mma<4, MB, BF16, true>(Q, 1, A1, acc, lb, 8);
+                if constexpr (DIRECT) {
+                    const u4_t T1[1] = {operand_of(A1[0])};
+                    half_mma<4, MB, BF16, true>(Q, 1, T1, acc, lb, 8);
+                } else {
+                    half_mma<4, MB, BF16, true>(Q, 1, A1, acc, lb, 8);
+                }
                 load_a(A1, ap + jstep);
                 __builtin_amdgcn_sched_barrier(0);
                 if (it < 10) GEMM_TRACE(6 + it);

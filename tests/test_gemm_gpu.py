@@ -95,6 +95,28 @@ def test_gemm_two_streams_residual_bias_every_workgroup_shape(monkeypatch, rows)
         assert rel_l2(y, ref) <= (TOL if act_dtype == torch.float16 else TOL_BF16)
 
 
+@pytest.mark.parametrize("M,N,K,gs", [(5, 256, 512, 128), (16, 512, 1024, 64), (33, 384, 1024, 256),
+                                      (130, 256, 2048, 128)])
+@pytest.mark.parametrize("act,lut", [(torch.float16, torch.float16), (torch.bfloat16, torch.float16),
+                                     (torch.bfloat16, torch.bfloat16)])
+def test_gemm_direct_activations_match_the_pre_pass(monkeypatch, M, N, K, gs, act, lut):
+    """With one 16-row block per wavefront the kernel reads A itself and transposes the
+    pieces in registers; FLUTE_GEMM_NO_DIRECT=1 sends the same call through the activation
+    pre-pass.  Both present identical operands, so the outputs are bit-identical; rows that
+    are not 16-byte aligned take the pre-pass by themselves."""
+    w = make_weight(N, K, 4, gs, seed=M + N, lut_dtype=lut, act_dtype=act, bias=True, device=DEV)
+    x = make_x(M, K, seed=17, dtype=act)
+    xd = x.to(DEV)
+    y = _dual(w, xd)
+    assert rel_l2(y.cpu(), _exact(w, x.to(lut)).to(act)) <= (TOL if act == torch.float16 else TOL_BF16)
+    monkeypatch.setenv("FLUTE_GEMM_NO_DIRECT", "1")
+    assert torch.equal(_dual(w, xd), y)
+    monkeypatch.delenv("FLUTE_GEMM_NO_DIRECT")
+    shifted = torch.zeros(M * K + 1, dtype=act, device=DEV)
+    shifted[1:] = xd.reshape(-1)
+    assert torch.equal(_dual(w, shifted[1:].reshape(M, K)), y)
+
+
 DUAL = [
     # M, N, K, bits, gs, bits2, rank, bias
     (8, 512, 1024, 4, 128, 1, 0, False),
