@@ -32,9 +32,10 @@ How each function is pinned (none of them by re-typing its own formula):
       adjoint(forward(x)) == x, norm preservation, per-segment independence
       (fht.py:19-35,137-167,740-771).
   rotation_signs
-      values in {-1,+1}; "parity unpinned" against upstream sign VALUES: no
-      upstream test or fixture records them, so only the generator recipe
-      (fht.py:105-115) is restated.
+      values pinned: upstream's recipe (fht.py:105-115) is randint(0, 2) on a CPU
+      generator seeded seed + 4242, i.e. the low bit of each word of the textbook
+      MT19937 stream; checked against numpy's MT19937 at K = 64, 4096, 12288 and
+      against the generator written out in the test (tests/test_oracle_math.py).
   pick_split
       the worked examples printed in src/kernel_gemv_splitk.cu:54-59.
 """

@@ -114,6 +114,57 @@ def test_hadamard_identities_and_segments():
     assert torch.equal(a[:, :64], b_[:, :64]) and not torch.equal(a[:, 64:], b_[:, 64:])
 
 
+def _mt19937_words(seed, count):
+    """The textbook MT19937 (Matsumoto & Nishimura 1998, init_genrand + genrand_int32),
+    written out so that the sign pin below does not rest on a library's word for it."""
+    mt = [0] * 624
+    mt[0] = seed & 0xFFFFFFFF
+    for i in range(1, 624):
+        mt[i] = (1812433253 * (mt[i - 1] ^ (mt[i - 1] >> 30)) + i) & 0xFFFFFFFF
+    out, idx = [], 624
+    while len(out) < count:
+        if idx >= 624:
+            for k in range(624):
+                y = (mt[k] & 0x80000000) | (mt[(k + 1) % 624] & 0x7FFFFFFF)
+                mt[k] = mt[(k + 397) % 624] ^ (y >> 1) ^ (0x9908B0DF if y & 1 else 0)
+            idx = 0
+        y = mt[idx]; idx += 1
+        y ^= y >> 11
+        y ^= (y << 7) & 0x9D2C5680
+        y ^= (y << 15) & 0xEFC60000
+        y ^= y >> 18
+        out.append(y)
+    return out
+
+
+@pytest.mark.parametrize("K", [64, 4096, 12288])
+@pytest.mark.parametrize("seed", [0, 7, 42])
+def test_rotation_sign_values_are_the_mt19937_low_bits(K, seed):
+    """Pins the VALUES of the sign vector.  Upstream draws
+    randint(0, 2, (K,)) * 2 - 1 from a CPU generator seeded seed + 4242
+    (fht.py:105-115); torch's CPU generator is MT19937 and randint(0, 2) keeps the low
+    bit of each 32-bit word, so sign k = 2 * (word_k & 1) - 1 of the textbook stream.
+    Checked against numpy's MT19937 at every size and against the generator written
+    out above on the first 700 words (past one state refill)."""
+    signs = O.rotation_signs(K, seed)
+    assert signs.dtype == torch.float32 and signs.shape == (K,)
+    bits = ((signs + 1) / 2).numpy().astype(np.int64)
+    words = np.random.RandomState(seed + 4242)._bit_generator.random_raw(K)
+    assert np.array_equal(bits, words & 1)
+    head = min(K, 700)
+    assert bits[:head].tolist() == [w & 1 for w in _mt19937_words(seed + 4242, head)]
+    # the product's own draw is the same vector
+    import fht
+    assert torch.equal(fht.rotation_signs(K, seed), signs)
+
+
+def test_mt19937_known_answer():
+    """genrand_int32 after init_genrand(5489) starts 3499211612, 581869302 (the
+    reference output of mt19937ar.c, also the C++11 default-seeded mt19937)."""
+    assert _mt19937_words(5489, 2) == [3499211612, 581869302]
+    assert _mt19937_words(5489, 10000)[-1] == 4123659995      # C++11 [rand.predef] 10000th value
+
+
 def test_fht_c_matches_numpy_bit_for_bit():
     path = os.path.join(ROOT, "oracle", "liboracle.so")
     if not os.path.exists(path):
