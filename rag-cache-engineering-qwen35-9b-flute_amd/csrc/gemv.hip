@@ -319,26 +319,25 @@ flute_status launch_fast4(Plan &plan, hipStream_t stream) {
     return FLUTE_OK;
 }
 
-// Loads a lane keeps in flight: the largest of 4, 3, 2 that divides the units of a
-// wavefront (no partial group in the K loop); 4 when the wavefronts differ or
-// nothing divides (that case runs the kernel's conservative tail).
+// Loads a lane keeps in flight in the lean kernel: 4 when that divides the loads of a
+// wavefront, else 2; 0 when the launch does not fit the kernel (the wavefronts would get
+// different or odd numbers of loads: two loads feed one matrix product).
 int pick_prefetch(const Plan &plan, int nw) {
     const int gpi = 64 >> plan.p.lpg_log2;
+    if (plan.p.gs_tiles % gpi) return 0;
     const int units = plan.p.gs_tiles / gpi;
-    int pf = env_int("FLUTE_GEMV4_PF", 0);
-    if (pf >= 2 && pf <= 4) return pf;
-    if (units % nw) return 4;
+    if (units % nw) return 0;
     const int u = units / nw;
-    for (int cand : {4, 3, 2})
-        if (u % cand == 0 || u < cand) return cand;
-    return 4;
+    if (u < 2 || (u & 1)) return 0;
+    const int pf = env_int("FLUTE_GEMV4_PF", 0);
+    if ((pf == 2 || pf == 4) && u % pf == 0) return pf;
+    return u % 4 == 0 ? 4 : 2;
 }
 
 template <int LPGL, int NW, bool BF16>
 flute_status launch_fast4_pf(Plan &plan, hipStream_t stream) {
     switch (pick_prefetch(plan, NW)) {
         case 2: return launch_fast4<LPGL, NW, 2, BF16>(plan, stream);
-        case 3: return launch_fast4<LPGL, NW, 3, BF16>(plan, stream);
         default: return launch_fast4<LPGL, NW, 4, BF16>(plan, stream);
     }
 }
@@ -368,8 +367,13 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
                            (plan.p.seg[0].xsrc == plan.p.seg[1].xsrc &&
                             plan.p.seg[0].signs == plan.p.seg[1].signs &&
                             plan.p.seg[0].awq == plan.p.seg[1].awq);
-    if (bits == 4 && one_group && one_input && es == 7 && (nw == 4 || nw == 8) &&
-        env_int("FLUTE_GEMV_NO_FAST", 0) == 0) {
+    // the lean kernel reads LUT rows through the scalar cache: dword-aligned LUTs only
+    bool luts_aligned = true;
+    for (int i = 0; i < plan.p.nsegs; ++i)
+        for (int st = 0; st < plan.p.seg[i].nstreams; ++st)
+            luts_aligned &= ((uintptr_t)plan.p.seg[i].st[st].lut & 3) == 0;
+    if (bits == 4 && one_group && one_input && es == 7 && (nw == 4 || nw == 8) && luts_aligned &&
+        pick_prefetch(plan, nw) != 0 && env_int("FLUTE_GEMV_NO_FAST", 0) == 0) {
         switch (plan.p.lpg_log2) {
             case 4: return launch_fast4_shape<4, BF16>(plan, nw, stream);
             case 5: return launch_fast4_shape<5, BF16>(plan, nw, stream);

@@ -1,24 +1,88 @@
 // Lean specialisation of the M = 1 LUT GEMV for the common case: every stream
 // 4 bits wide and one LUT group per 128-row tile (group_size >= 128).  Same
-// ownership, lane mapping, table format and K-split protocol as gemv_kernel.h;
-// the row-slice width, the wavefront count and the table stride are template
-// constants so that the prologue and the per-load overhead shrink to a few
-// dozen instructions.
+// ownership, table format and K-split protocol as gemv_kernel.h; what differs is
+// how a looked-up weight pair meets the activations.
+//
+// Matrix cores instead of dot products.  The K loop is bound by the rate at which
+// a CU issues LDS lookups (about one wavefront lookup per nanosecond), so every
+// vector instruction next to a lookup costs time.  The looked-up pairs are
+// therefore fed to v_mfma_f32_16x16x32 as they come out of the table:
+//   * lane L = (kg, rb, kt) = (L >> 4, (L >> 2) & 3, L & 3) reads quarter kt of
+//     chunk (cg0 + cgl, kg) of tile gsub, where rb = (gsub, cgl) splits by the
+//     slice width.  Four lanes with equal L >> 2 read 64 contiguous bytes and a
+//     wavefront load covers 1 KB of whole 64-byte pieces.
+//   * a 16-byte load holds, per row (v, d) of the lane's eight rows, the bytes
+//     s2 = 0, 1 = four consecutive-pair k values.  Two loads give eight k values
+//     per row: one A operand of the 16x16x32 product per (v, d), whose matrix row
+//     is i = (rb, kt) and whose k block is kg.
+//   * the k values of a lane depend on kt, which is part of the matrix row.  The B
+//     operand therefore carries, in column j = (rb', kt'), the activations of
+//     quarter kt' of tile gsub(rb'): the product D[i][j] is the wanted partial sum
+//     where kt' = kt and gsub(rb') = gsub(rb), and the other columns are ignored.
+//     The matrix cores are idle otherwise, so the unused columns cost nothing.
+//   * D[i][j] sits in lane (j + 16 * (i >> 2)), register i & 3: the lanes with
+//     rb' = rb keep register kt', a quad sum folds kt', and one LDS exchange folds
+//     the tiles of a load and the wavefronts.
+// Per weight pair this leaves two address instructions and the lookup; the
+// multiply-accumulate and the cross-lane reduction of the dot-product form are gone.
+//
+// The LUT row (32 bytes) comes through the scalar cache, so it does not queue
+// behind the index loads of the other workgroups of the CU in the vector memory
+// pipe; index loads are non-temporal (read once).
 #pragma once
 
 #include "gemv_kernel.h"
 
 namespace flute {
 
+typedef _Float16 gv_h8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 gv_bf8_t __attribute__((ext_vector_type(8)));
+typedef float gv_f4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t gv_u4_t __attribute__((ext_vector_type(4)));
+
+template <bool BF16>
+__device__ __forceinline__ gv_f4_t gv_mfma(gv_u4_t a, gv_u4_t b, gv_f4_t c) {
+    if constexpr (BF16) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gv_bf8_t, a),
+                                                       __builtin_bit_cast(gv_bf8_t, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(gv_h8_t, a),
+                                                      __builtin_bit_cast(gv_h8_t, b), c, 0, 0, 0);
+    }
+}
+
+// Sixteen index bytes, read once: non-temporal, so they do not displace the
+// activations and LUT rows that every workgroup shares from the caches.
+__device__ __forceinline__ uint4 load_idx16(const uint8_t *p) {
+    typedef const __attribute__((address_space(1))) gv_u4_t *GlobalQuad;       // global, not flat
+    const gv_u4_t v = __builtin_nontemporal_load((GlobalQuad)(uintptr_t)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// One LUT row of sixteen 16-bit values through the scalar cache (the pointer is
+// wavefront-uniform and 4-byte aligned).
+__device__ __forceinline__ void load_lut_row(const uint16_t *lut, uint32_t (&d)[8]) {
+    typedef const __attribute__((address_space(4))) uint32_t *ConstWord;
+    ConstWord p = (ConstWord)(const void *)lut;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) d[i] = p[i];
+}
+
+// Value c (0..15) of a LUT row held as eight uniform dwords.
+__device__ __forceinline__ uint32_t lut_value(const uint32_t (&d)[8], int c) {
+    const int i = c >> 1;
+    const uint32_t a = (i & 1) ? d[1] : d[0], b = (i & 1) ? d[3] : d[2];
+    const uint32_t e = (i & 1) ? d[5] : d[4], f = (i & 1) ? d[7] : d[6];
+    const uint32_t ab = (i & 2) ? b : a, ef = (i & 2) ? f : e;
+    const uint32_t w = (i & 4) ? ef : ab;
+    return (c & 1) ? (w >> 16) : (w & 0xffffu);
+}
+
 // LPGL = log2(lanes per 64-k tile) = log2(2 * rows per workgroup): 4, 5, 6.
-// NW   = wavefronts per workgroup.
-// PF   = index loads a lane keeps in flight (2, 3 or 4).  A few loads per
-//        wavefront, refilled as they are consumed, serve every wavefront of the grid
-//        in turn; a deep queue (a wavefront's whole K range requested at once) is
-//        served wavefront by wavefront, and the last ones served start their
-//        arithmetic when the memory stream is already over.  The host picks the
-//        largest PF that divides the units of a wavefront, so that the K loop has no
-//        partial group.
+// NW   = wavefronts per workgroup (4 or 8).
+// PF   = index loads a lane keeps in flight (2 or 4).  The host picks a PF that
+//        divides the loads of a wavefront, which it makes equal for all wavefronts
+//        and even (two loads feed one matrix product).
 // The table stride is 128 bytes (32 replicas of a 4-byte entry, 32 KB): three
 // four-wavefront workgroups fit a CU.
 template <int LPGL, int NW, int PF, bool BF16>
@@ -30,13 +94,15 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     constexpr int GPI = 64 >> LPGL;                 // 64-k tiles per wavefront load
     constexpr int RW = LPG >> 1;                    // rows per workgroup
     constexpr int SPT = 128 / RW;                   // row slices per tile
+    constexpr int SH = LPGL - 4;                    // bits of rb that pick the chunk group
     constexpr int XV = 2;                           // 16-byte activation loads per thread
-    constexpr int PF0 = 1;                          // index loads issued ahead of the table build
+    constexpr int PF0 = 2;                          // index loads issued ahead of the table build
     constexpr int STRIDE = 1 << ES;                 // table bytes per entry
     constexpr int CHUNKS = STRIDE / 16;             // 16-byte pieces of one entry's replicas
     constexpr int SHARES = NT / 256;                // threads per table entry
     constexpr int CPT = CHUNKS / SHARES;            // pieces written per thread
     static_assert(NT >= 256, "one thread per table entry at least");
+    static_assert(PF % 2 == 0 && PF >= PF0, "loads are consumed in pairs");
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     warm_kernargs<(int)sizeof(GemvParams)>(kp);
@@ -51,31 +117,29 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const int tid = threadIdx.x;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int L = tid & 63;
-    const int gsub = L >> LPGL;
-    const int l = L & (LPG - 1);
+    const int kg = L >> 4, rb = (L >> 2) & 3, kt = L & 3;
+    const int gsub = rb >> SH;                      // tile of the load this lane reads
+    const int cgl = rb & ((1 << SH) - 1);           // chunk group inside the row slice
     const int sl = (int)blockIdx.x - kp->seg[si0].col0;
     const int t = sl / SPT;
     const int cg0 = (sl % SPT) * (RW >> 3);
     const int s = blockIdx.y;
     const int g_lo = s * p.gs_tiles;
     const int units = p.gs_tiles / GPI;
-    const int my_units = units > w ? (units - w + NW - 1) / NW : 0;
+    const int my_units = units / NW;                // the host makes this exact, even, >= PF
     const int k0 = g_lo * 64, kc = p.gs_tiles * 64;
     const int G = p.K >> 6;
 
     uint16_t *xs = (uint16_t *)(lds + p.lds_x);
-    const uint32_t *xs32 = (const uint32_t *)xs;
-    float *red = (float *)(lds + p.lds_red);        // [2][NW][32] row sums
+    float *red = (float *)(lds + p.lds_red);        // [2][NW][4][8] partial row sums
 
     // lane-constant pieces of the addresses
     const uint32_t unit_bytes = GPI * 4096u;
-    const uint32_t lane0 = (uint32_t)gsub * 4096u + (uint32_t)cg0 * 256u + (uint32_t)l * 16u +
-                           (uint32_t)w * unit_bytes;
+    const uint32_t lane0 = (uint32_t)gsub * 4096u + (uint32_t)(cg0 + cgl) * 256u +
+                           (uint32_t)kg * 64u + (uint32_t)kt * 16u + (uint32_t)w * unit_bytes;
     constexpr uint32_t step = NW * GPI * 4096u;
-    const int xi = gsub * 32 + (l & 3) * 8 + ((l >> 2) & 3) + w * (GPI * 32);
     // Lookup addresses are formed as absolute LDS addresses, so the (zero) base of
-    // the dynamic LDS block is folded into the per-lane replica offset once
-    // instead of being added after every v_perm.
+    // the dynamic LDS block is folded into the per-lane replica offset once.
     typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     const uint32_t slot = lds_base + (uint32_t)(L & 31) * 4u;
@@ -95,65 +159,65 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         qr = st.q + ((size_t)t * G + g_lo) * 4096u;
         lutp = st.lut + ((size_t)grp << 4);
     };
-    // A wavefront with fewer than PF loads re-reads the first unit of the K range
-    // (always present) into the registers it will not consume: every load below is
-    // unconditional, so the compiler knows how many are in flight at each point and
-    // waits for exactly the one it needs.  One conditional load in a loop makes it
-    // wait for all of them at the loop head, which serialises the memory stream and
-    // the arithmetic.
     // Index loads are addressed as (uniform base + unit offset) in scalar registers
     // plus one lane-constant 32-bit offset, so no per-load address lives in vector
-    // registers.
-    auto unit_load = [&](const uint8_t *qr, int unit) -> uint4 {
-        const uint8_t *base = unit < my_units ? qr + (size_t)unit * step
-                                              : qr - (size_t)w * unit_bytes;
-        return *(const uint4 *)(base + lane0);
-    };
-    auto first_units = [&](const uint8_t *qr, uint4 (&qq)[PF]) {
+    // registers; every load is unconditional, so the compiler knows how many are in
+    // flight at each point and waits for exactly the ones a product needs.
+    auto first_units = [&](const uint8_t *qr, uint4 (&qq)[PF], int from) {
 #pragma unroll
         for (int n = 0; n < PF; ++n) {
-            qq[n] = unit_load(qr, n);
-            __builtin_amdgcn_sched_barrier(0);      // issue order = consumption order
+            if (n >= from) {
+                qq[n] = load_idx16(qr + (size_t)n * step + lane0);
+                __builtin_amdgcn_sched_barrier(0);  // issue order = consumption order
+            }
         }
     };
 
     // Paired table: entry e -> {lut[e & 15], lut[e >> 4]}, replicated over the stride;
     // 16 bytes per store, starting at a lane-dependent piece so that a wavefront
     // spreads over the banks.
-    auto write_table = [&](uint32_t lo_, uint32_t hi_) {
-        const uint32_t v = lo_ | (hi_ << 16);
+    auto write_table = [&](const uint32_t (&row)[8]) {
+        const uint32_t v = lut_value(row, e_own & 15) | (lut_value(row, e_own >> 4) << 16);
         const uint4 v4 = make_uint4(v, v, v, v);
         uint8_t *ent = lds + e_own * STRIDE + share * (CPT * 16);
 #pragma unroll
         for (int k = 0; k < CPT; ++k) *(uint4 *)(ent + (((k + tid) & (CPT - 1)) << 4)) = v4;
     };
 
-    FLUTE_TRACE(0);
+    // Activations in operand order: for load unit u (GPI tiles) the 8 bytes
+    // {k, k+1, k+8, k+9} of (kg, tile, kt) lie together, so a lane reads the B half of
+    // a product as one 8-byte LDS word.  Eight consecutive activations (one tile,
+    // quarter and s2; kg = 0..3) scatter to four such words.
+    auto stage8 = [&](int j, uint4 v) {
+        const int g = j >> 6, kk = j & 63;
+        const int u = g / GPI, gs_ = g % GPI;
+        uint32_t *dst = (uint32_t *)xs + u * (32 * GPI) + ((gs_ * 4 + (kk >> 4)) << 1) + ((kk >> 3) & 1);
+        dst[0] = v.x;
+        dst[GPI * 8] = v.y;
+        dst[GPI * 16] = v.z;
+        dst[GPI * 24] = v.w;
+    };
+
     // Wavefront priority falls as a workgroup advances: 3 in the prologue, 2 while
     // there is more to stream, 1 in the last group, 0 from the fold on.  A SIMD holds
     // one wavefront of each resident workgroup and serves the oldest first; without
-    // this the workgroup that arrived last on a CU lags through the whole launch and
-    // ends more than a microsecond after the first.
+    // this the workgroup that arrived last on a CU lags through the whole launch.
     __builtin_amdgcn_s_setprio(3);
-    // ---- first pass: activations, LUT values and the first index bytes.  The order
-    //      of the loads is the order they are needed in, and the scheduler is kept
-    //      from changing it: a wait for an early load also waits for everything
-    //      issued before it. ---------------------------------------------------------
     int so = 0, si = 0;
     const uint8_t *qrow;
     const uint16_t *lut;
     pass_ptrs(0, 0, qrow, lut);
+    uint32_t lrow[8];
+    load_lut_row(lut, lrow);
     const uint16_t *staged_x = kp->seg[si0].xsrc ? kp->seg[si0].xsrc : p.x;
     const float *staged_signs = kp->seg[si0].signs, *staged_awq = kp->seg[si0].awq;
     const bool x_direct = staged_signs == nullptr;  // plain copy
     const bool x_short = kc <= XV * NT * 8;         // uniform
     uint4 q[PF];
-    uint32_t lo, hi;
     if (x_direct && x_short) {
-        // The usual case.  A few index loads go out ahead of the table build so that
-        // the memory stream starts early; the rest follow once the table is written.
-        // (All of them at once would put every other workgroup's activation and LUT
-        // loads behind a full batch of index bytes in the CU's memory queue.)
+        // The usual case: activations first, then two index loads, the table (its LUT
+        // row arrives through the scalar cache meanwhile), the rest of the loads, and
+        // the activations into LDS.
         uint4 xv[XV];
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
@@ -161,76 +225,58 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             xv[i] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
         }
         __builtin_amdgcn_sched_barrier(0);
-        lo = lut[e_own & 15];
-        hi = lut[e_own >> 4];
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int n = 0; n < PF0; ++n) {
-            q[n] = unit_load(qrow, n);
+            q[n] = load_idx16(qrow + (size_t)n * step + lane0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        FLUTE_TRACE(1);
+        write_table(lrow);
+        first_units(qrow, q, PF0);
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
             const int j = (i * NT + tid) * 8;
-            if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(xv[i], p.act_bf16);
-        }
-        write_table(lo, hi);
-#pragma unroll
-        for (int n = PF0; n < PF; ++n) {
-            q[n] = unit_load(qrow, n);
-            __builtin_amdgcn_sched_barrier(0);
+            if (j < kc) stage8(j, to_compute_type<BF16>(xv[i], p.act_bf16));
         }
     } else if (x_direct) {
-        // A long K range: everything the table and the staged activations need is
-        // fetched and written first (the index registers carry the activations
-        // meanwhile), then the index loads start.
+        // A long K range: the index registers carry the activations first.
 #pragma unroll
         for (int n = 0; n < PF; ++n) {
             const int j = (n * NT + tid) * 8;
             q[n] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
         }
         __builtin_amdgcn_sched_barrier(0);
-        lo = lut[e_own & 15];
-        hi = lut[e_own >> 4];
-        __builtin_amdgcn_sched_barrier(0);
-        FLUTE_TRACE(1);
 #pragma unroll
         for (int n = 0; n < PF; ++n) {
             const int j = (n * NT + tid) * 8;
-            if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(q[n], p.act_bf16);
+            if (j < kc) stage8(j, to_compute_type<BF16>(q[n], p.act_bf16));
         }
         for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8)
-            *(uint4 *)(xs + j) =
-                to_compute_type<BF16>(*(const uint4 *)(staged_x + k0 + j), p.act_bf16);
-        write_table(lo, hi);
+            stage8(j, to_compute_type<BF16>(*(const uint4 *)(staged_x + k0 + j), p.act_bf16));
+        write_table(lrow);
         __builtin_amdgcn_sched_barrier(0);
-        first_units(qrow, q);
+        first_units(qrow, q, 0);
     } else {
-        // A rotated input: the LUT values and the first index loads travel while the
-        // rotation runs.
-        lo = lut[e_own & 15];
-        hi = lut[e_own >> 4];
-        __builtin_amdgcn_sched_barrier(0);
+        // A rotated input: the rotation leaves the slice in natural order; the first
+        // index loads travel while it runs.
 #pragma unroll
         for (int n = 0; n < PF0; ++n) {
-            q[n] = unit_load(qrow, n);
+            q[n] = load_idx16(qrow + (size_t)n * step + lane0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        FLUTE_TRACE(1);
         stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
-        write_table(lo, hi);
+        write_table(lrow);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int n = PF0; n < PF; ++n) {
-            q[n] = unit_load(qrow, n);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        first_units(qrow, q, PF0);
     }
 
-    float acc[8];
+    gv_f4_t acc[8];
 #pragma unroll
-    for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
+    for (int a = 0; a < 8; ++a) acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+
+    const uint2 *xs64 = (const uint2 *)xs;
+    const uint32_t *xs32 = (const uint32_t *)xs;
+    const int xoff = (kg * GPI + gsub) * 4 + kt;    // operand order: 8-byte word of this lane
+    const int xnat = gsub * 32 + kt * 8 + kg;       // natural order: first dword of this lane
 
     for (bool first = true;; first = false) {
         const int sg = so == 1 ? 1 : si0;
@@ -238,14 +284,12 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             // every output of the launch reads the same staged activations (the host
             // sends launches whose outputs differ in input or rotation to the general
             // kernel), so only the table changes between passes
-            write_table(lo, hi);
+            write_table(lrow);
         }
 
-        // ---- the pass after this one: its LUT values are fetched now and its first
-        //      index loads replace this pass's last ones as they are consumed, so the
-        //      memory stream does not stop between passes.  Without a next pass the
-        //      same LUT values are read again (harmless, and keeps the load count
-        //      unconditional). -----------------------------------------------------------
+        // ---- the pass after this one: its LUT row is fetched now and its first index
+        //      loads replace this pass's last ones as they are consumed, so the memory
+        //      stream does not stop between passes. -----------------------------------
         int nso = so, nsi = si + 1;
         if (nsi == kp->seg[sg].nstreams) {
             nsi = 0;
@@ -254,114 +298,102 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         const bool has_next = nso < nout;
         const uint8_t *qnext = qrow;
         const uint16_t *lutn = lut;
-        if (has_next) pass_ptrs(nso, nsi, qnext, lutn);
-        __builtin_amdgcn_sched_barrier(0);
-        lo = lutn[e_own & 15];
-        hi = lutn[e_own >> 4];
-        __builtin_amdgcn_sched_barrier(0);
+        if (has_next) {
+            pass_ptrs(nso, nsi, qnext, lutn);
+            load_lut_row(lutn, lrow);
+        }
         __syncthreads();
-#ifdef FLUTE_GEMV_TRACE
-        if (first) FLUTE_TRACE(2); else if (so == 1 && si == 0) FLUTE_TRACE(7);
-#endif
 
         // ---- K loop -----------------------------------------------------------------
-        // One unit = one 16-byte load of this lane.  Its sixteen table lookups go out
-        // together and are consumed together, so the LDS latency is paid once per
-        // load, not once per dword.
-        auto lookups = [&](const uint4 &qv, uint32_t (&e)[4][4]) {
+        // One step = two 16-byte loads of this lane = 32 lookups and 8 matrix products.
+        auto lookups = [&](const uint4 &qv, uint32_t (&e)[16]) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const uint32_t wv = v == 0 ? qv.x : v == 1 ? qv.y : v == 2 ? qv.z : qv.w;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {       // byte j: d = j >> 1, s2 = j & 1
-                    e[v][j] = *(LdsWord)((((wv >> (8 * j)) & 0xffu) << ES) + slot);
-                }
+                for (int j = 0; j < 4; ++j)         // byte j: d = j >> 1, s2 = j & 1
+                    e[v * 4 + j] = *(LdsWord)((((wv >> (8 * j)) & 0xffu) << ES) + slot);
             }
         };
-        auto dots = [&](const uint32_t (&e)[4][4], int m) {
-            const int xo = xi + m * (NW * GPI * 32);
-            const uint32_t xa = xs32[xo];
-            const uint32_t xb = xs32[xo + 4];
+        auto operand_b = [&](int m0, int m1) -> gv_u4_t {
+            const int u0 = w + m0 * NW, u1 = w + m1 * NW;
+            if (x_direct) {
+                const uint2 xa = xs64[u0 * (16 * GPI) + xoff], xb = xs64[u1 * (16 * GPI) + xoff];
+                return (gv_u4_t){xa.x, xa.y, xb.x, xb.y};
+            }
+            const int a0 = u0 * (32 * GPI) + xnat, a1 = u1 * (32 * GPI) + xnat;
+            return (gv_u4_t){xs32[a0], xs32[a0 + 4], xs32[a1], xs32[a1 + 4]};
+        };
+        auto products = [&](const uint32_t (&e0)[16], const uint32_t (&e1)[16], gv_u4_t B) {
 #pragma unroll
             for (int v = 0; v < 4; ++v)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[v * 2 + (j >> 1)] =
-                        dot2<BF16>(e[v][j], (j & 1) ? xb : xa, acc[v * 2 + (j >> 1)]);
+                for (int d = 0; d < 2; ++d) {
+                    const gv_u4_t A = {e0[v * 4 + 2 * d], e0[v * 4 + 2 * d + 1], e1[v * 4 + 2 * d],
+                                       e1[v * 4 + 2 * d + 1]};
+                    acc[v * 2 + d] = gv_mfma<BF16>(A, B, acc[v * 2 + d]);
+                }
         };
         int nb = 0;
         __builtin_amdgcn_s_setprio(2);
         for (; nb + 2 * PF <= my_units; nb += PF) {          // every refill exists
 #pragma unroll
-            for (int n = 0; n < PF; ++n) {
-                uint32_t e[4][4];
-                lookups(q[n], e);
+            for (int n = 0; n < PF; n += 2) {
+                uint32_t e0[16], e1[16];
+                const gv_u4_t B = operand_b(nb + n, nb + n + 1);
+                lookups(q[n], e0);
+                lookups(q[n + 1], e1);
                 // pinned: the scheduler would otherwise sink all refills to the end of
                 // the body, draining the prefetch queue once per group
                 __builtin_amdgcn_sched_barrier(0);
-                q[n] = *(const uint4 *)(qrow + (size_t)(nb + n + PF) * step + lane0);
+                q[n] = load_idx16(qrow + (size_t)(nb + n + PF) * step + lane0);
+                q[n + 1] = load_idx16(qrow + (size_t)(nb + n + 1 + PF) * step + lane0);
                 __builtin_amdgcn_sched_barrier(0);
-                dots(e, nb + n);
+                products(e0, e1, B);
             }
         }
         if (!has_next) __builtin_amdgcn_s_setprio(1);
-        if (nb + PF == my_units && has_next) {                // a full last group, refilled
-#pragma unroll                                                //   from the next pass
-            for (int n = 0; n < PF; ++n) {
-                uint32_t e[4][4];
-                lookups(q[n], e);
-                __builtin_amdgcn_sched_barrier(0);
-                q[n] = *(const uint4 *)(qnext + (size_t)n * step + lane0);
-                __builtin_amdgcn_sched_barrier(0);
-                dots(e, nb + n);
-            }
-        } else if (nb + PF >= my_units) {                     // the last group, no refills
+        // the last group (my_units is a multiple of PF), refilled from the next pass when
+        // there is one; two copies so that the loads of each are unconditional
+        if (has_next) {
 #pragma unroll
-            for (int n = 0; n < PF; ++n) {
-                if (nb + n < my_units) {                      // uniform within the wavefront
-                    uint32_t e[4][4];
-                    lookups(q[n], e);
-                    dots(e, nb + n);
-                }
+            for (int n = 0; n < PF; n += 2) {
+                uint32_t e0[16], e1[16];
+                const gv_u4_t B = operand_b(nb + n, nb + n + 1);
+                lookups(q[n], e0);
+                lookups(q[n + 1], e1);
+                __builtin_amdgcn_sched_barrier(0);
+                q[n] = load_idx16(qnext + (size_t)n * step + lane0);
+                q[n + 1] = load_idx16(qnext + (size_t)(n + 1) * step + lane0);
+                __builtin_amdgcn_sched_barrier(0);
+                products(e0, e1, B);
             }
-            if (has_next) first_units(qnext, q);
-        } else {                                              // a partial group follows
-            for (; nb < my_units; nb += PF) {
+        } else {
 #pragma unroll
-                for (int n = 0; n < PF; ++n) {
-                    const int m = nb + n;
-                    if (m < my_units) {
-                        uint32_t e[4][4];
-                        lookups(q[n], e);
-                        if (m + PF < my_units)
-                            q[n] = *(const uint4 *)(qrow + (size_t)(m + PF) * step + lane0);
-                        dots(e, m);
-                    }
-                }
+            for (int n = 0; n < PF; n += 2) {
+                uint32_t e0[16], e1[16];
+                const gv_u4_t B = operand_b(nb + n, nb + n + 1);
+                lookups(q[n], e0);
+                lookups(q[n + 1], e1);
+                products(e0, e1, B);
             }
-            __builtin_amdgcn_s_waitcnt(0x0F70);                // vmcnt(0): see below
-            if (has_next) first_units(qnext, q);
         }
-#ifdef FLUTE_GEMV_TRACE
-        if (!has_next) FLUTE_TRACE(3); else if (first) FLUTE_TRACE(6);
-#endif
 
         if (!has_next) __builtin_amdgcn_s_setprio(0);
-        // ---- end of an output: fold the lanes that share rows ------------------------
+        // ---- end of an output: D[i][j] with i = (rb, kt) in (lane >> 4, register) and
+        //      j = (rb', kt') in lane & 15.  The lanes with rb' == rb keep register kt';
+        //      a quad sum folds kt'. ----------------------------------------------------
         if (nso != so) {
+            const bool keep = rb == kg;             // here L >> 4 is the matrix row block
 #pragma unroll
             for (int a = 0; a < 8; ++a) {
-                float v = row16_sum(acc[a]);
-                if constexpr (LPGL <= 5) v += __shfl_xor(v, 32);
-                if constexpr (LPGL == 4) v += __shfl_xor(v, 16);
-                acc[a] = v;
+                float v = kt == 0 ? acc[a][0] : kt == 1 ? acc[a][1] : kt == 2 ? acc[a][2] : acc[a][3];
+                v = keep ? v : 0.0f;
+                v = dpp_add<0xB1>(v);               // quad_perm [1,0,3,2]
+                v = dpp_add<0x4E>(v);               // quad_perm [2,3,0,1]
+                if (keep && kt == 0) red[(so * NW + w) * 32 + rb * 8 + a] = v;
+                acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
             }
-            if (L < LPG && (L & 15) == 0) {
-#pragma unroll
-                for (int a = 0; a < 8; ++a) red[(so * NW + w) * 32 + (L >> 4) * 8 + a] = acc[a];
-            }
-#pragma unroll
-            for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
         }
         if (!has_next) break;
         __syncthreads();                            // the table region is rewritten next
@@ -371,12 +403,12 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         lut = lutn;
     }
     __syncthreads();
-    FLUTE_TRACE(4);
 
-    // ---- one thread per owned row --------------------------------------------------
+    // ---- one thread per owned row: fold the wavefronts and the tiles of a load ------
     if (tid >= RW && p.split == 1) return;
     const bool owner = tid < RW;
-    const int n = t * 128 + row_of(cg0 + (tid >> 3), tid & 7);
+    const int cgl_o = tid >> 3, a_o = tid & 7;
+    const int n = t * 128 + row_of(cg0 + cgl_o, a_o);
     float yv[2] = {0.0f, 0.0f};
     if (owner) {
 #pragma unroll
@@ -384,7 +416,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             if (so >= nout) break;
             float y = 0.0f;
 #pragma unroll
-            for (int ww = 0; ww < NW; ++ww) y += red[(so * NW + ww) * 32 + tid];
+            for (int ww = 0; ww < NW; ++ww)
+#pragma unroll
+                for (int gb = 0; gb < GPI; ++gb)
+                    y += red[(so * NW + ww) * 32 + ((gb << SH) | cgl_o) * 8 + a_o];
             yv[so] = y;
         }
     }
@@ -449,7 +484,6 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         if (p.silu_mul) y = (yv[0] / (1.0f + expf(-yv[0]))) * yv[1];
         kp->seg[si0].out[n] = round_act(y, p.act_bf16);
     }
-    FLUTE_TRACE(5);
 }
 
 }  // namespace flute
