@@ -206,6 +206,23 @@ flute_status flute_validate(const flute_linear *w, int mode);
 /* Release the per-device split-K workspaces (also done at process exit). */
 void flute_release_workspaces(void);
 
+/*
+ * The launchers read their tuning and test knobs (FLUTE_GEMV_RW, FLUTE_GEMV_WAVES,
+ * FLUTE_GEMV_TABLE_LOG2, FLUTE_GEMV_PREROTATE, FLUTE_GEMV4_PF, FLUTE_GEMV_NO_FAST,
+ * FLUTE_GEMM_ROWS, FLUTE_GEMM_NO_PERM, FLUTE_GEMM_KSPLIT, FLUTE_GEMM_NO_DIRECT,
+ * FLUTE_FHT_STEPS) from the environment once per process; this re-reads them.
+ */
+void flute_reload_tuning(void);
+
+/*
+ * What a workspace request does, as pure host arithmetic (usable without a GPU):
+ * 0 = the buffers held are large enough, 1 = they grow (hipMalloc), 2 = refused with
+ * FLUTE_ERR_INVALID because the stream is being captured into a graph and the buffers
+ * would have to grow.  Sizes in elements.
+ */
+int flute_workspace_decision(int64_t have_floats, int64_t need_floats, int64_t have_ints,
+                             int64_t need_ints, int capturing);
+
 #ifdef __cplusplus
 }
 #endif

@@ -448,8 +448,8 @@ flute_status fht_launch(const void *x, int64_t ldx, const float *signs, const fl
     // 21.0 us for one row, 52.6 us against 40.3 us for 1024 rows).  FLUTE_FHT_STEPS = 0, 2
     // or 4 forces a variant (tuning and test knob).
     int steps = wide ? (rows <= 512 ? 4 : 0) : 2;
-    if (const char *e = getenv("FLUTE_FHT_STEPS")) {
-        const int v = atoi(e);
+    {
+        const int v = tuning().fht_steps;
         if (v == 0 || v == 2 || v == 4) steps = v;
     }
     if (steps == 0)

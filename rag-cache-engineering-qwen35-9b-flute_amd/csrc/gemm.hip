@@ -29,8 +29,8 @@ struct GemmShape {
 // CU's LDS, so one workgroup per CU is resident.  FLUTE_GEMM_ROWS = 16, 32, 64 or 128
 // forces the shape (a tuning and test knob, like FLUTE_GEMV_RW).
 GemmShape choose_gemm_shape(int M, int tiles, int64_t index_bytes) {
-    if (const char *e = getenv("FLUTE_GEMM_ROWS")) {
-        const int v = atoi(e);
+    {
+        const int v = tuning().gemm_rows;
         if (v == 16) return {1, 8, 1, 1};
         if (v == 32) return {2, 8, 1, 1};
         if (v == 64) return {4, 8, 1, 1};
@@ -62,22 +62,6 @@ flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t st
     return FLUTE_OK;
 }
 
-#ifdef FLUTE_GEMM_DEV_MINIMAL
-// Development builds: only the 4-bit fp16 M > 64 kernel, to keep compile time short.
-template <bool BF16>
-flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 grid, int lds,
-                               hipStream_t stream) {
-    if (!BF16 && p.nstreams == 1 && p.bits[0] == 4 && p.rep_log2[0] == 6) {
-        if (s.mb == 1 && p.A8) return launch_gemm<1, 8, 1, false, 4, true, true>(p, grid, lds, stream);
-        if (s.mb == 1) return launch_gemm<1, 8, 1, false, 4, true>(p, grid, lds, stream);
-        if (s.mb == 2) return launch_gemm<2, 8, 1, false, 4, true>(p, grid, lds, stream);
-        if (s.mw == 1) return launch_gemm<4, 8, 1, false, 4, true>(p, grid, lds, stream);
-        return launch_gemm<4, 4, 2, false, 4, true>(p, grid, lds, stream);
-    }
-    set_error("flute_gemm: development build without this kernel");
-    return FLUTE_ERR_UNSUPPORTED;
-}
-#else
 template <int MB, int KW, int MW, bool BF16>
 flute_status launch_gemm_bits(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
     if (p.nstreams == 1) {
@@ -111,7 +95,6 @@ flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 gri
     return launch_gemm_bits<4, 4, 2, BF16>(p, grid, lds, stream);
 }
 
-#endif
 
 // LDS plan of one launch: pair tables (+ staging on the fast path), sized against the
 // reduction tree and the totals tile that reuse the same memory afterwards.
@@ -122,7 +105,7 @@ flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 gri
 int plan_lds(GemmParams &p, const GemmShape &shape) {
     const int ngrp = p.gs >= 128 ? 1 : 128 / p.gs;
     const bool perm = p.nstreams == 1 && p.bits[0] == 4 && ngrp <= 2 &&
-                      getenv("FLUTE_GEMM_NO_PERM") == nullptr;
+                      !tuning().gemm_no_perm;
     const int table_budget = (shape.mb == 1 ? 64 : 96) * 1024 / p.nstreams;
     int lds_tables = 0;
     for (int s = 0; s < p.nstreams; ++s) {
@@ -213,8 +196,8 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     while (units * ksplit * 2 <= cap && ksplit * 2 <= max_split &&
            p.G / (ksplit * 2) >= shape.kw * 2)
         ksplit *= 2;
-    if (const char *e = getenv("FLUTE_GEMM_KSPLIT")) {
-        const int v = atoi(e);
+    {
+        const int v = tuning().gemm_ksplit;
         if (v >= 1 && v <= p.G) ksplit = v;
     }
     p.gper = (p.G + ksplit - 1) / ksplit;
@@ -246,9 +229,9 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     {
         const int ngrp = w->group_size >= 128 ? 1 : 128 / w->group_size;
         const bool fast = p.nstreams == 1 && w->b1 == 4 && ngrp <= 2 &&
-                          getenv("FLUTE_GEMM_NO_PERM") == nullptr;
+                          !tuning().gemm_no_perm;
         if (shape.mb == 1 && fast && !w->signs && ((uintptr_t)A & 15) == 0 && lda % 8 == 0 &&
-            getenv("FLUTE_GEMM_NO_DIRECT") == nullptr) {
+            !tuning().gemm_no_direct) {
             p.A8 = (const u4_t *)A;
             p.lda8 = lda / 8;
             p.a_bf16 = act_dtype == FLUTE_BF16;
@@ -289,9 +272,6 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
         p.xb = xb;
     }
 
-#ifdef FLUTE_GEMM_TRACE
-    if (const char *e = getenv("FLUTE_GEMM_TRACE_PTR")) p.trace = (unsigned long long *)strtoull(e, nullptr, 10);
-#endif
     // Two streams with four blocks per wavefront: one launch per stream through the
     // single-stream kernels (the two-stream kernel does not fit the register file at
     // that size); both write partial tiles and the last workgroup of the second launch

@@ -62,9 +62,6 @@ struct GemmParams {
     const u4_t *A8;        // direct mode: A itself, rows of lda8 16-byte pieces, no pre-pass
     int64_t lda8;
     int a_bf16;            // dtype of A in direct mode
-#ifdef FLUTE_GEMM_TRACE
-    unsigned long long *trace;   // [workgroup][16] timestamps, development builds only
-#endif
 };
 
 // Activation pre-pass: Ap[g][j][mb][lane][slot] in the LUT's 16-bit type.
@@ -146,16 +143,6 @@ __device__ __forceinline__ void ws_load16x4(const float *p0, const float *p1, co
         : "memory");
 }
 
-#ifdef FLUTE_GEMM_TRACE
-#define GEMM_TRACE(slot)                                                                    \
-    do {                                                                                    \
-        if (p.trace && threadIdx.x == 0)                                                    \
-            p.trace[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16 + \
-                    (slot)] = wall_clock64();                                               \
-    } while (0)
-#else
-#define GEMM_TRACE(slot) do {} while (0)
-#endif
 
 template <bool BF16>
 __device__ __forceinline__ f4_t mfma16(u4_t w, u4_t a, f4_t acc) {
@@ -291,7 +278,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     const int wx = rho >> 3;
     const int th = wx * 32 + (rho & 7) * 4 + kg;
 
-    GEMM_TRACE(0);
     const int gbeg = z * p.gper, gend = min(p.G, gbeg + p.gper);
     const bool active = mb0 < p.mblk_total;            // whole wavefront
     const int g0 = gbeg + kw;
@@ -389,7 +375,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         }
     }
     __syncthreads();
-    GEMM_TRACE(1);
 
     f4_t acc[MB][8];
 #pragma unroll
@@ -454,7 +439,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 if (left > 1) tp += qstep;
                 load_tile();                              // second tile (or a harmless reload)
             }
-            int it = 0;
             while (left > 0) {
                 stage_read();                             // this tile's chunk
                 __builtin_amdgcn_sched_barrier(0);
@@ -481,8 +465,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 }
                 load_a(A1, ap + jstep);
                 __builtin_amdgcn_sched_barrier(0);
-                if (it < 10) GEMM_TRACE(6 + it);
-                ++it;
                 --left;
             }
         } else if constexpr (B1 > 0) {
@@ -567,9 +549,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 
     // ---- tree over the KW wavefronts of one m group, through LDS ------------------
     f4_t *red = (f4_t *)smem;                           // slot = [MB*8][64] f4
-    GEMM_TRACE(2);
     __syncthreads();                                    // tables are dead from here
-    GEMM_TRACE(3);
 #pragma unroll
     for (int step = KW / 2; step >= 1; step >>= 1) {
         if (kw >= step && kw < 2 * step) {
@@ -590,7 +570,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         __syncthreads();
     }
 
-    GEMM_TRACE(4);
     // ---- totals of the workgroup as a row-major fp32 tile in LDS --------------------
     constexpr int ROWS = MW * MB * 16;                  // rows of C this workgroup owns
     constexpr int LDT = 128 + 4;                        // padded row: conflict-free both ways
@@ -703,7 +682,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             }
         }
     }
-    GEMM_TRACE(5);
 }
 
 }  // namespace flute

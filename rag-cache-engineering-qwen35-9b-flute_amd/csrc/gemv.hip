@@ -9,16 +9,11 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 namespace flute {
 
 namespace {
-
-int env_int(const char *name, int fallback) {
-    const char *e = std::getenv(name);
-    if (!e || !*e) return fallback;
-    return std::atoi(e);
-}
 
 int entries_log2(int bits) { return bits == 3 ? 6 : 8; }
 int entry_bytes_log2(int bits) { return bits >= 3 ? 2 : (bits == 2 ? 3 : 4); }
@@ -53,7 +48,7 @@ struct Plan {
 // at K = 2048...16384; e.g. N = 1024, K = 4096: 5.0 us against 6.7 us split four
 // ways).  A caller's explicit split is honoured.
 void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *waves) {
-    int best_rw = env_int("FLUTE_GEMV_RW", 0);
+    int best_rw = tuning().gemv_rw;
     if (best_rw != 8 && best_rw != 16 && best_rw != 32) {
         // The narrowest slices whose grid is still resident at once (three four-wavefront
         // workgroups per CU): a second round of workgroups costs far more than wider
@@ -82,7 +77,7 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
     }
     *rw = best_rw;
     *split = sp;
-    int wv = env_int("FLUTE_GEMV_WAVES", 0);
+    int wv = tuning().gemv_waves;
     if (wv != 1 && wv != 2 && wv != 4 && wv != 8) {
         // Eight wavefronts when each still has two loads or more and the grid is at most
         // one workgroup per CU, or two per CU of eight-row workgroups with a long K range
@@ -155,7 +150,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     // LDS: tables/scratch | x slice | row sums.  The table stride is the largest
     // that still lets the whole grid be resident at once (one round of
     // workgroups), since a second round repeats the start-up latency.
-    int budget = env_int("FLUTE_GEMV_TABLE_LOG2", 0);
+    int budget = tuning().gemv_table_log2;
     if (budget < 12 || budget > 17) {
         long wgs = 0;
         for (int i = 0; i < (silu_mul ? 1 : count); ++i) wgs += (long)(segs[i].N / rw) * split;
@@ -191,7 +186,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
         // front measured slower still (a dependent launch costs more than that), so it
         // stays an opt-in.
         const bool prerotate = w.signs != nullptr && w.R == 0 &&
-                               env_int("FLUTE_GEMV_PREROTATE", 0) != 0;
+                               tuning().gemv_prerotate != 0;
         if (w.R > 0 || prerotate) {
             // the residual needs x . resB[r] before any row can finish: computed by a
             // small kernel in front, on the rotated input when the weight is rotated
@@ -284,12 +279,6 @@ flute_status launch_typed(Plan &plan, hipStream_t stream) {
                                             (int)kLdsPerCU));
         attr_done = true;
     }
-#ifdef FLUTE_GEMV_TRACE
-    {
-        const char *e = std::getenv("FLUTE_GEMV_TRACE_PTR");
-        plan.p.trace = e ? (unsigned long long *)std::strtoull(e, nullptr, 0) : nullptr;
-    }
-#endif
     dim3 grid(plan.grid_x, plan.p.split);
     hipLaunchKernelGGL((gemv_kernel<BF16, BFIX>), grid, dim3(plan.threads), plan.lds_bytes, stream,
                        plan.p);
@@ -306,12 +295,6 @@ flute_status launch_fast4(Plan &plan, hipStream_t stream) {
                                             (int)kLdsPerCU));
         attr_done = true;
     }
-#ifdef FLUTE_GEMV_TRACE
-    {
-        const char *e = std::getenv("FLUTE_GEMV_TRACE_PTR");
-        plan.p.trace = e ? (unsigned long long *)std::strtoull(e, nullptr, 0) : nullptr;
-    }
-#endif
     dim3 grid(plan.grid_x, plan.p.split);
     hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, PF, BF16>), grid, dim3(NW * 64), plan.lds_bytes,
                        stream, plan.p);
@@ -329,7 +312,7 @@ int pick_prefetch(const Plan &plan, int nw) {
     if (units % nw) return 0;
     const int u = units / nw;
     if (u < 2 || (u & 1)) return 0;
-    const int pf = env_int("FLUTE_GEMV4_PF", 0);
+    const int pf = tuning().gemv4_pf;
     if ((pf == 2 || pf == 4) && u % pf == 0) return pf;
     return u % 4 == 0 ? 4 : 2;
 }
@@ -373,7 +356,7 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         for (int st = 0; st < plan.p.seg[i].nstreams; ++st)
             luts_aligned &= ((uintptr_t)plan.p.seg[i].st[st].lut & 3) == 0;
     if (bits == 4 && one_group && one_input && es == 7 && (nw == 4 || nw == 8) && luts_aligned &&
-        pick_prefetch(plan, nw) != 0 && env_int("FLUTE_GEMV_NO_FAST", 0) == 0) {
+        pick_prefetch(plan, nw) != 0 && tuning().gemv_no_fast == 0) {
         switch (plan.p.lpg_log2) {
             case 4: return launch_fast4_shape<4, BF16>(plan, nw, stream);
             case 5: return launch_fast4_shape<5, BF16>(plan, nw, stream);
@@ -389,14 +372,28 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
     }
 }
 
-flute_status launch(Plan &plan, int act_dtype, hipStream_t stream) {
+// Scratch memory a launch needs beyond its operands: partial sums of a K split, tickets,
+// residual coefficients, pre-rotated inputs.
+struct ScratchNeed {
+    size_t floats, ints;
+};
+ScratchNeed scratch_need(const Plan &plan) {
+    if (!(plan.p_floats || plan.npre)) return {0, 0};
+    const size_t xb_pad = (plan.xb_floats + 3) & ~(size_t)3;
+    return {plan.p_floats + xb_pad + (plan.xrot_halves + 1) / 2 + 64, (size_t)plan.total_tickets + 1};
+}
+
+// fixed_base/fixed_tickets: caller-provided scratch (the allocation-free entry point);
+// null = the library's per-device workspace, grown on demand.
+flute_status launch(Plan &plan, int act_dtype, hipStream_t stream, float *fixed_base = nullptr,
+                    int *fixed_tickets = nullptr) {
     if (plan.p_floats || plan.npre) {
         const size_t xb_pad = (plan.xb_floats + 3) & ~(size_t)3;
-        const size_t floats = plan.p_floats + xb_pad + (plan.xrot_halves + 1) / 2 + 64;
-        float *base = nullptr;
-        int *tickets = nullptr;
-        flute_status st = get_workspace(floats, (size_t)plan.total_tickets + 1, stream, &base,
-                                        &tickets);
+        const ScratchNeed need = scratch_need(plan);
+        float *base = fixed_base;
+        int *tickets = fixed_tickets;
+        flute_status st = FLUTE_OK;
+        if (!base) st = get_workspace(need.floats, need.ints, stream, &base, &tickets);
         if (st != FLUTE_OK) return st;
         plan.p.P = base;
         plan.p.tickets = tickets;

@@ -84,9 +84,6 @@ struct GemvParams {
     int fht_block;          // > 0: equal rotation blocks of this many columns
     int lds_x;              // LDS byte offsets
     int lds_red;
-#ifdef FLUTE_GEMV_TRACE
-    unsigned long long *trace;   // [workgroup][8] timestamps, development builds only
-#endif
 };
 
 // Reads one dword of every 64-byte line of the kernel-argument block with
@@ -103,15 +100,6 @@ __device__ __forceinline__ void warm_kernargs(const void *kernargs) {
     asm volatile("" ::"s"(seen));
 }
 
-#ifdef FLUTE_GEMV_TRACE
-#define FLUTE_TRACE(slot)                                                              \
-    do {                                                                               \
-        if (p.trace && threadIdx.x == 0)                                               \
-            p.trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8 + (slot)] = wall_clock64(); \
-    } while (0)
-#else
-#define FLUTE_TRACE(slot) do {} while (0)
-#endif
 
 // ---- small device helpers ---------------------------------------------------
 
@@ -954,7 +942,6 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     StreamRegs<BF> first;
     const uint16_t *x0 = sg.xsrc ? sg.xsrc : p.x;
     const bool x_ahead = BFIX != 0 && sg.signs == nullptr;      // uniform
-    FLUTE_TRACE(0);
     if (x_ahead) {
         uint4 xv[XV];
 #pragma unroll
@@ -963,7 +950,6 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
             xv[i] = *(const uint4 *)(x0 + k0 + (j < kc ? j : 0));
         }
         if constexpr (BFIX != 0) stream_issue<BF>(p, sg, sg.st[0], gm, first);
-        FLUTE_TRACE(1);
         uint16_t *xs = (uint16_t *)(lds + p.lds_x);
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
@@ -976,7 +962,6 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     } else {
         stage_x<BF16>(p, x0, sg.signs, sg.awq, lds, k0, kc, gm.tid, gm.nthreads);
         if constexpr (BFIX != 0) stream_issue<BF>(p, sg, sg.st[0], gm, first);
-        FLUTE_TRACE(1);
     }
     const uint16_t *staged_x = x0;
     const float *staged_signs = sg.signs, *staged_awq = sg.awq;
@@ -990,7 +975,6 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
             staged_signs = og.signs;
             staged_awq = og.awq;
         }
-        FLUTE_TRACE(2);
         float acc[8];
 #pragma unroll
         for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
@@ -1001,10 +985,8 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
                     stream_tables<BF>(st, gm, lds, first);
                     stream_issue_rest<BF>(gm, first);
                     __syncthreads();
-                    FLUTE_TRACE(3);
                     stream_loop<BF, BF16>(p, og, st, gm, lds, first, acc);
                     __syncthreads();
-                    FLUTE_TRACE(4);
                 }
             } else {
                 run_stream_any<BF16, BFIX>(p, og, st, gm, lds, acc);
@@ -1107,7 +1089,6 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
         if (p.silu_mul) y = (yv[0] / (1.0f + expf(-yv[0]))) * yv[1];
         sg.out[n] = round_act(y, p.act_bf16);
     }
-    FLUTE_TRACE(5);
 }
 
 // Residual coefficients: xb[r] = sum_k x[k] * resB[r][k] in fp32, one workgroup

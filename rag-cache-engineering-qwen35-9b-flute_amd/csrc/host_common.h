@@ -15,8 +15,28 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who);
 // tickets are zeroed once at allocation and every kernel leaves them at zero.
 // One workspace per device: launches that use it must be ordered on one stream
 // (the same contract as upstream include/flute/gemv_host.h:31-38).
+// When the buffers must grow while `stream` is being captured into a graph the call is
+// refused (FLUTE_ERR_INVALID): an allocation and the clearing of fresh tickets cannot be
+// part of a capture.  Warm the shape up outside the capture first.
 flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float **P,
                            int **tickets);
+
+// What get_workspace does for a request, as pure host arithmetic: 0 = the buffers are
+// large enough, 1 = they grow, 2 = growth refused because the stream is capturing.
+int workspace_decision(size_t have_floats, size_t need_floats, size_t have_ints, size_t need_ints,
+                       bool capturing);
+
+// Tuning and test knobs of the launchers, read from the environment once per process
+// (flute_reload_tuning re-reads them): FLUTE_GEMV_RW, FLUTE_GEMV_WAVES,
+// FLUTE_GEMV_TABLE_LOG2, FLUTE_GEMV_PREROTATE, FLUTE_GEMV4_PF, FLUTE_GEMV_NO_FAST,
+// FLUTE_GEMM_ROWS, FLUTE_GEMM_NO_PERM, FLUTE_GEMM_KSPLIT, FLUTE_GEMM_NO_DIRECT,
+// FLUTE_FHT_STEPS.  Unset or empty = 0, except fht_steps = -1.
+struct Tuning {
+    int gemv_rw, gemv_waves, gemv_table_log2, gemv_prerotate, gemv4_pf, gemv_no_fast;
+    int gemm_rows, gemm_no_perm, gemm_ksplit, gemm_no_direct;
+    int fht_steps;
+};
+const Tuning &tuning();
 
 // The Walsh-Hadamard rotation of flute_fht with row strides, and optionally with its
 // output written in the operand order of the LUT GEMM (the image the GEMM's activation

@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <atomic>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -90,12 +91,30 @@ static std::mutex g_ws_mu;
 static std::unordered_map<int, Workspace> g_ws;
 static std::vector<void *> g_retired;   // outgrown buffers, freed at release
 
+int workspace_decision(size_t have_floats, size_t need_floats, size_t have_ints, size_t need_ints,
+                       bool capturing) {
+    if (have_floats >= need_floats && have_ints >= need_ints) return 0;
+    return capturing ? 2 : 1;
+}
+
 flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float **P,
                            int **tickets) {
     int dev = 0;
     FLUTE_HIP_CHECK(hipGetDevice(&dev));
     std::lock_guard<std::mutex> guard(g_ws_mu);
     Workspace &ws = g_ws[dev];
+    if (ws.floats < floats || ws.ints < ints) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        FLUTE_HIP_CHECK(hipStreamIsCapturing(stream, &cap));
+        if (workspace_decision(ws.floats, floats, ws.ints, ints,
+                               cap != hipStreamCaptureStatusNone) == 2) {
+            set_error("workspace: this call needs %zu B of partial sums and %zu tickets, more than the "
+                      "%zu B / %zu held, and the stream is being captured: an allocation cannot be "
+                      "part of a graph. Run the same call once outside the capture first",
+                      floats * sizeof(float), ints, ws.floats * sizeof(float), ws.ints);
+            return FLUTE_ERR_INVALID;
+        }
+    }
     if (ws.floats < floats) {
         size_t want = ws.floats ? ws.floats : (size_t)1 << 20;
         while (want < floats) want *= 2;
@@ -126,6 +145,43 @@ flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float
     return FLUTE_OK;
 }
 
+static Tuning g_tuning;
+static std::atomic<bool> g_tuning_ready{false};
+static std::mutex g_tuning_mu;
+
+static int env_or(const char *name, int fallback) {
+    const char *e = std::getenv(name);
+    if (!e || !*e) return fallback;
+    return std::atoi(e);
+}
+
+static void read_tuning() {
+    Tuning t;
+    t.gemv_rw = env_or("FLUTE_GEMV_RW", 0);
+    t.gemv_waves = env_or("FLUTE_GEMV_WAVES", 0);
+    t.gemv_table_log2 = env_or("FLUTE_GEMV_TABLE_LOG2", 0);
+    t.gemv_prerotate = env_or("FLUTE_GEMV_PREROTATE", 0);
+    t.gemv4_pf = env_or("FLUTE_GEMV4_PF", 0);
+    t.gemv_no_fast = env_or("FLUTE_GEMV_NO_FAST", 0);
+    t.gemm_rows = env_or("FLUTE_GEMM_ROWS", 0);
+    t.gemm_no_perm = std::getenv("FLUTE_GEMM_NO_PERM") != nullptr;
+    t.gemm_ksplit = env_or("FLUTE_GEMM_KSPLIT", 0);
+    t.gemm_no_direct = std::getenv("FLUTE_GEMM_NO_DIRECT") != nullptr;
+    t.fht_steps = env_or("FLUTE_FHT_STEPS", -1);
+    g_tuning = t;
+}
+
+const Tuning &tuning() {
+    if (!g_tuning_ready.load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> guard(g_tuning_mu);
+        if (!g_tuning_ready.load(std::memory_order_relaxed)) {
+            read_tuning();
+            g_tuning_ready.store(true, std::memory_order_release);
+        }
+    }
+    return g_tuning;
+}
+
 }  // namespace flute
 
 extern "C" {
@@ -138,6 +194,18 @@ const char *flute_target_arch(void) { return "gfx950"; }
 
 flute_status flute_validate(const flute_linear *w, int mode) {
     return flute::validate_linear(w, mode, "flute_validate");
+}
+
+void flute_reload_tuning(void) {
+    std::lock_guard<std::mutex> guard(flute::g_tuning_mu);
+    flute::read_tuning();
+    flute::g_tuning_ready.store(true, std::memory_order_release);
+}
+
+int flute_workspace_decision(int64_t have_floats, int64_t need_floats, int64_t have_ints,
+                             int64_t need_ints, int capturing) {
+    return flute::workspace_decision((size_t)have_floats, (size_t)need_floats, (size_t)have_ints,
+                                     (size_t)need_ints, capturing != 0);
 }
 
 void flute_release_workspaces(void) {

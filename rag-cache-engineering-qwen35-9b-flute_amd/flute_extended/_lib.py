@@ -67,6 +67,8 @@ SYMBOLS = {
     "flute_gemv_lds_bytes": (ctypes.c_int64, [_LP, _I]),
     "flute_validate": (_I, [_LP, _I]),
     "flute_release_workspaces": (None, []),
+    "flute_reload_tuning": (None, []),
+    "flute_workspace_decision": (_I, [ctypes.c_int64] * 4 + [_I]),
 }
 
 if not os.path.exists(LIB_PATH):

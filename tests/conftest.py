@@ -24,3 +24,22 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def tuning_env(monkeypatch):
+    """Set one of the library's tuning variables for a test.  The library reads them once
+    per process, so every change is followed by flute_reload_tuning(), also when the
+    environment is restored."""
+    from flute_extended import _lib
+
+    def set_var(name, value):
+        if value is None:
+            monkeypatch.delenv(name, raising=False)
+        else:
+            monkeypatch.setenv(name, value)
+        _lib.lib.flute_reload_tuning()
+
+    yield set_var
+    monkeypatch.undo()
+    _lib.lib.flute_reload_tuning()

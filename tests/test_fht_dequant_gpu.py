@@ -59,11 +59,11 @@ def test_fht_block_mode_and_round_trip():
 
 @pytest.mark.parametrize("steps", ["0", "2", "4"])
 @pytest.mark.parametrize("K", [1536, 4096, 12288, 24576])
-def test_fht_every_kernel_variant_bit_exact(monkeypatch, steps, K):
+def test_fht_every_kernel_variant_bit_exact(tuning_env, steps, K):
     """Segments are transformed through the LDS buffer, or up to 4096 / 8192 columns in
     registers with one LDS pass; the library picks by K and the number of rows.  Each
-    variant forced in turn (FLUTE_FHT_STEPS, read per call) must give the reference's bits."""
-    monkeypatch.setenv("FLUTE_FHT_STEPS", steps)
+    variant forced in turn (FLUTE_FHT_STEPS) must give the reference's bits."""
+    tuning_env("FLUTE_FHT_STEPS", steps)
     signs = O.rotation_signs(K, 7)
     for dtype in (torch.float32, torch.bfloat16):
         x = make_x(3, K, seed=K, dtype=dtype)

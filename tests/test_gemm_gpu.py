@@ -70,11 +70,11 @@ def test_gemm_single_stream_fp16(M, N, K, bits, gs):
 
 @pytest.mark.parametrize("rows", ["16", "32", "64", "128"])
 @pytest.mark.parametrize("M,N,K,bits,gs", [c for c in SINGLE if c[0] > 16])
-def test_gemm_every_workgroup_shape(monkeypatch, rows, M, N, K, bits, gs):
+def test_gemm_every_workgroup_shape(tuning_env, rows, M, N, K, bits, gs):
     """The library picks the rows of A per workgroup (16, 32, 64 or 128) from M, N and K; at
     the small N of these cases it would always pick 16, so each shape is forced in turn
-    (FLUTE_GEMM_ROWS, read per call) and must give the oracle's result."""
-    monkeypatch.setenv("FLUTE_GEMM_ROWS", rows)
+    (FLUTE_GEMM_ROWS) and must give the oracle's result."""
+    tuning_env("FLUTE_GEMM_ROWS", rows)
     w = make_weight(N, K, bits, gs, seed=M + N + K + bits, device=DEV)
     x = make_x(M, K, seed=11)
     y = fx.qgemm_per_group_lut(x.to(DEV), w["blob_d"], w["lut_d"], bitwidth=bits, group_size=gs,
@@ -83,8 +83,8 @@ def test_gemm_every_workgroup_shape(monkeypatch, rows, M, N, K, bits, gs):
 
 
 @pytest.mark.parametrize("rows", ["16", "32", "64", "128"])
-def test_gemm_two_streams_residual_bias_every_workgroup_shape(monkeypatch, rows):
-    monkeypatch.setenv("FLUTE_GEMM_ROWS", rows)
+def test_gemm_two_streams_residual_bias_every_workgroup_shape(tuning_env, rows):
+    tuning_env("FLUTE_GEMM_ROWS", rows)
     M, N, K = 40, 256, 1024
     for lut_dtype, act_dtype in ((torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16)):
         w = make_weight(N, K, 4, 128, seed=7, bits2=2, rank=8, bias=True, lut_dtype=lut_dtype,
@@ -99,7 +99,7 @@ def test_gemm_two_streams_residual_bias_every_workgroup_shape(monkeypatch, rows)
                                       (130, 256, 2048, 128)])
 @pytest.mark.parametrize("act,lut", [(torch.float16, torch.float16), (torch.bfloat16, torch.float16),
                                      (torch.bfloat16, torch.bfloat16)])
-def test_gemm_direct_activations_match_the_pre_pass(monkeypatch, M, N, K, gs, act, lut):
+def test_gemm_direct_activations_match_the_pre_pass(tuning_env, M, N, K, gs, act, lut):
     """With one 16-row block per wavefront the kernel reads A itself and transposes the
     pieces in registers; FLUTE_GEMM_NO_DIRECT=1 sends the same call through the activation
     pre-pass.  Both present identical operands, so the outputs are bit-identical; rows that
@@ -109,9 +109,9 @@ def test_gemm_direct_activations_match_the_pre_pass(monkeypatch, M, N, K, gs, ac
     xd = x.to(DEV)
     y = _dual(w, xd)
     assert rel_l2(y.cpu(), _exact(w, x.to(lut)).to(act)) <= (TOL if act == torch.float16 else TOL_BF16)
-    monkeypatch.setenv("FLUTE_GEMM_NO_DIRECT", "1")
+    tuning_env("FLUTE_GEMM_NO_DIRECT", "1")
     assert torch.equal(_dual(w, xd), y)
-    monkeypatch.delenv("FLUTE_GEMM_NO_DIRECT")
+    tuning_env("FLUTE_GEMM_NO_DIRECT", None)
     shifted = torch.zeros(M * K + 1, dtype=act, device=DEV)
     shifted[1:] = xd.reshape(-1)
     assert torch.equal(_dual(w, shifted[1:].reshape(M, K)), y)

@@ -208,3 +208,42 @@ def test_fused_block_rotation_is_bit_identical_to_rotate_then_gemv(block, dtype)
     assert torch.equal(fused, _run(w, xr.cpu()))
     xo = O.block_fht_reference(x, block, signs)
     assert rel_l2(fused.cpu(), _exact(w, xo).to(dtype)) <= (TOL if dtype == torch.float16 else 4e-3)
+
+
+def test_workspace_growth_is_refused_under_graph_capture():
+    """A K split needs the library workspace.  When that would have to be allocated while
+    the stream is being captured, the call is refused (an allocation and the clearing of
+    fresh tickets cannot be graph nodes); after a warm-up outside the capture the same call
+    is captured and replays."""
+    import ctypes
+    from flute_extended import _lib
+    w = make_weight(512, 2048, seed=41, device=DEV)
+    x = make_x(1, 2048, seed=42).to(DEV)
+    d = _lib.FluteLinear()
+    d.q1, d.lut1, d.q1_bytes = w["blob_d"].data_ptr(), w["lut_d"].data_ptr(), w["blob_d"].numel()
+    d.N, d.K, d.b1, d.group_size, d.lut_rows, d.lut_dtype = 512, 2048, 4, 128, 4, _lib.F16
+    y = torch.zeros(1, 512, dtype=torch.float16, device=DEV)
+    torch.cuda.synchronize()
+    _lib.lib.flute_release_workspaces()                 # nothing held: the next split call must allocate
+    call = lambda: _lib.lib.flute_gemv(ctypes.byref(d), x.data_ptr(), y.data_ptr(), _lib.F16, 4,
+                                       torch.cuda.current_stream().cuda_stream)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        with torch.cuda.graph(g, stream=s):
+            y.zero_()
+            status = call()
+            message = _lib.last_error()
+    assert status == _lib.FLUTE_ERR_INVALID and "captured" in message
+    assert call() == 0                                  # warm-up outside a capture allocates
+    torch.cuda.synchronize()
+    want = y.clone()
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s):
+        with torch.cuda.graph(g2, stream=s):
+            assert call() == 0
+    y.zero_()
+    g2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, want)

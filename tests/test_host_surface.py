@@ -269,3 +269,36 @@ def test_fused_mlp_falls_through_on_unfusable_inputs():
     assert torch.equal(y, ref)
     assert mlp._merge_state is None                                 # fp32 input: never built
     assert mlp._build_state(torch.device("cpu"), torch.float16)["reason"] == "reference member"
+
+
+def test_workspace_decision_refuses_growth_under_capture():
+    """The branch get_workspace takes: enough room -> nothing happens (capturing or not);
+    too little -> grow outside a capture, refuse inside one."""
+    from flute_extended import _lib
+    dec = _lib.lib.flute_workspace_decision
+    assert dec(1 << 20, 1000, 1 << 14, 10, 0) == 0
+    assert dec(1 << 20, 1000, 1 << 14, 10, 1) == 0
+    assert dec(1 << 20, (1 << 20) + 1, 1 << 14, 10, 0) == 1
+    assert dec(1 << 20, (1 << 20) + 1, 1 << 14, 10, 1) == 2
+    assert dec(0, 0, 0, 1, 1) == 2 and dec(0, 0, 0, 0, 1) == 0
+
+
+def test_tuning_is_read_once_and_on_reload(monkeypatch):
+    """Tuning variables do not reach the library until flute_reload_tuning(): the split
+    policy (pure host arithmetic) shows which value is in force."""
+    from flute_extended import _lib
+    before = _lib.lib.flute_gemv_lds_bytes
+    w = _lib.FluteLinear()
+    w.q1 = w.lut1 = 16
+    w.N, w.K, w.b1, w.group_size, w.lut_rows, w.lut_dtype = 1024, 4096, 4, 128, 8, _lib.F16
+    w.q1_bytes = 1024 * 4096 // 2
+    base = before(w, 1)
+    monkeypatch.setenv("FLUTE_GEMV_TABLE_LOG2", "13")
+    assert before(w, 1) == base                         # not re-read per call
+    _lib.lib.flute_reload_tuning()
+    try:
+        assert before(w, 1) != base
+    finally:
+        monkeypatch.undo()
+        _lib.lib.flute_reload_tuning()
+    assert before(w, 1) == base
