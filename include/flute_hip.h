@@ -101,6 +101,22 @@ flute_status flute_gemv(const flute_linear *w, const void *x, void *y,
                         int act_dtype, int split, void *stream);
 
 /*
+ * flute_gemv for callers that cannot allocate (code under HIP graph capture, serving
+ * loops and harnesses that forbid hipMalloc).  No counterpart upstream.  Same operands,
+ * same kernels and bit-identical results; what flute_gemv takes from the library's
+ * growing workspace (partial sums and tickets of a K split, residual coefficients, the
+ * pre-rotated input of a rotated weight with a residual) lives in a fixed 2 MiB array
+ * that is part of the code object: each device the library runs on holds its own copy
+ * until the process ends.  The call allocates nothing and frees nothing.  A launch whose
+ * scratch exceeds the array (more than 520192 floats or 4096 tickets: roughly
+ * split * (N + R) + R + K/2 floats, N/8 tickets) is refused with FLUTE_ERR_UNSUPPORTED.
+ * Every call on a device shares that device's array: calls that overlap on one device
+ * (two streams, or a replaying graph next to eager calls) race; order them.
+ */
+flute_status flute_gemv_noalloc(const flute_linear *w, const void *x, void *y,
+                                int act_dtype, int split, void *stream);
+
+/*
  * Merged gate+up GEMV with the SiLU*mul epilogue, M = 1:
  *   h[n] = silu(gate(x)[n]) * up(x)[n],   silu(v) = v / (1 + exp(-v)), fp32,
  * one rounding to act_dtype.  Replaces qgemm_gemv_mlp (src/bindings.cpp:378-384,

@@ -424,6 +424,44 @@ flute_status launch(Plan &plan, int act_dtype, hipStream_t stream, float *fixed_
     return plan.lut_bf16 ? launch_width<true>(plan, stream) : launch_width<false>(plan, stream);
 }
 
+// ---- the allocation-free variant's scratch ------------------------------------------
+// One fixed array per device, part of the code object: held from the time the library is
+// loaded on a device until the process ends.  Layout: [tickets: kNoAllocTickets ints]
+// [partial sums, residual coefficients, pre-rotated input: the rest as floats].
+constexpr size_t kNoAllocBytes = (size_t)2 << 20;
+constexpr size_t kNoAllocTickets = 4096;
+constexpr size_t kNoAllocFloats = (kNoAllocBytes - kNoAllocTickets * sizeof(int)) / sizeof(float);
+constexpr int kMaxDevices = 64;
+
+static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
+
+__global__ void zero_ints_kernel(int *dst, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = 0;
+}
+
+static std::mutex g_scratch_mu;
+static unsigned char *g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of this device's copy of the array (the array's name is a host-side
+// stand-in, not a device address): resolved once per device, with that device current.
+flute_status noalloc_scratch(unsigned char **out) {
+    int dev = 0;
+    FLUTE_HIP_CHECK(hipGetDevice(&dev));
+    FLUTE_REQUIRE(dev >= 0 && dev < kMaxDevices, FLUTE_ERR_UNSUPPORTED,
+                  "flute_gemv_noalloc: device ordinal %d beyond %d", dev, kMaxDevices);
+    std::lock_guard<std::mutex> guard(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        unsigned char *ptr = nullptr;
+        FLUTE_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        FLUTE_REQUIRE(ptr != nullptr, FLUTE_ERR_HIP,
+                      "flute_gemv_noalloc: the scratch array has no address on device %d", dev);
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return FLUTE_OK;
+}
+
 }  // namespace
 
 }  // namespace flute
@@ -439,6 +477,37 @@ flute_status flute_gemv(const flute_linear *w, const void *x, void *y, int act_d
     flute_status st = make_plan(w, 1, x, outs, act_dtype, split, 0, "flute_gemv", &plan);
     if (st != FLUTE_OK) return st;
     return launch(plan, act_dtype, (hipStream_t)stream);
+}
+
+flute_status flute_gemv_noalloc(const flute_linear *w, const void *x, void *y, int act_dtype,
+                                int split, void *stream) {
+    Plan plan;
+    void *outs[1] = {y};
+    flute_status st = make_plan(w, 1, x, outs, act_dtype, split, 0, "flute_gemv_noalloc", &plan);
+    if (st != FLUTE_OK) return st;
+    const ScratchNeed need = scratch_need(plan);
+    FLUTE_REQUIRE(need.floats <= kNoAllocFloats && need.ints <= kNoAllocTickets,
+                  FLUTE_ERR_UNSUPPORTED,
+                  "flute_gemv_noalloc: this launch needs %zu B of scratch and %zu tickets; the fixed "
+                  "array holds %zu B and %zu tickets (N=%d, K=%d, R=%d, split=%d). Use flute_gemv, "
+                  "or a smaller split",
+                  need.floats * sizeof(float), need.ints, kNoAllocFloats * sizeof(float),
+                  kNoAllocTickets, w->N, w->K, w->R, plan.p.split);
+    if (need.floats == 0) return launch(plan, act_dtype, (hipStream_t)stream);
+    unsigned char *ptr = nullptr;
+    st = noalloc_scratch(&ptr);
+    if (st != FLUTE_OK) return st;
+    int *tickets = (int *)ptr;
+    float *base = (float *)(ptr + kNoAllocTickets * sizeof(int));
+    if (plan.p.split > 1) {
+        // the array keeps the last call's contents: tickets must start at zero (a fill
+        // kernel, not a memset node, so that the call can be captured into a graph)
+        const int n = (int)need.ints;
+        hipLaunchKernelGGL(zero_ints_kernel, dim3((n + 255) / 256), dim3(256), 0,
+                           (hipStream_t)stream, tickets, n);
+        FLUTE_HIP_CHECK(hipGetLastError());
+    }
+    return launch(plan, act_dtype, (hipStream_t)stream, base, tickets);
 }
 
 flute_status flute_gemv_mlp(const flute_linear *gate, const flute_linear *up, const void *x,

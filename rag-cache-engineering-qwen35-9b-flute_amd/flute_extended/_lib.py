@@ -56,6 +56,7 @@ SYMBOLS = {
     "flute_last_error": (ctypes.c_char_p, []),
     "flute_target_arch": (ctypes.c_char_p, []),
     "flute_gemv": (_I, [_LP, _P, _P, _I, _I, _P]),
+    "flute_gemv_noalloc": (_I, [_LP, _P, _P, _I, _I, _P]),
     "flute_gemv_mlp": (_I, [_LP, _LP, _P, _P, _I, _I, _P]),
     "flute_gemv_multi": (_I, [_LP, _I, _P, ctypes.POINTER(_P), _I, _I, _P]),
     "flute_mlp_block": (_I, [_LP, _LP, _LP, _P, _P, _P, _I, _P]),
