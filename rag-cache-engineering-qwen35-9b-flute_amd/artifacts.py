@@ -192,12 +192,20 @@ def _read_stream2(meta: Dict, artifacts_dir: str, ctx: str, N: int, K: int, bitw
 
 
 def _awq_for(meta: Dict, awq_scales: Optional[Dict]):
-    """(scale tensor or None, fold order or None) for one tensor record."""
-    rec = meta.get("awq") or {}
-    s = None
-    if awq_scales:
-        s = awq_scales.get(meta.get("var")) or awq_scales.get(meta.get("name"))
-    return s, rec.get("fold_order")
+    """(scale tensor or None, fold order or None) for one tensor record
+    (scripts/palettized_modules.py:2590-2615 upstream).  `awq_scales` maps consumer
+    tensor names to (K,) tensors; a tensor without an entry is unscaled.  QKV components
+    are resolved on the fused record (they share the module input and the one fold).
+    The fold order is the record's awq.fold_order, else its rotation.order, else None
+    (the constructor then assumes the legacy rotate-then-AWQ order)."""
+    if not awq_scales:
+        return None, None
+    key = meta.get("var") or meta.get("name")
+    s = awq_scales.get(key)
+    if s is None:
+        return None, None
+    fold = (meta.get("awq") or {}).get("fold_order") or (meta.get("rotation") or {}).get("order")
+    return s, fold
 
 
 def _build(meta, artifacts_dir, ctx, shape, residual, reference, verify_sha, awq_s, fold, bias):

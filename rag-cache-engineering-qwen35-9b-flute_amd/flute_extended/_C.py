@@ -536,10 +536,12 @@ def gemv_lds_bytes(N: int, K: int, bitwidth: int, bitwidth2: int, group_size: in
 
 def embedding_gather(ids, indices, lut, N: int, K: int, bitwidth: int, group_size: int,
                      indices2=None, lut2=None, bitwidth2: int = 0, resB=None, resA=None,
-                     signs=None, rot_block: int = 0):
+                     signs=None, rot_block: int = 0, check_ids: bool = True):
     """Rows `ids` of a palettized table in the LUT's dtype (PalettizedEmbedding.forward,
     scripts/palettized_modules.py:2298-2335 upstream).  ids: any integer tensor on the
-    table's device; ids outside [0, N) raise, as upstream's range check does."""
+    table's device; ids outside [0, N) raise, as upstream's range check does
+    (check_ids=False skips that host read for a caller that has checked already or
+    is capturing a graph: the kernel then writes a row of zeros for such an id)."""
     who = "embedding_gather"
     if ids.dtype not in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8):
         _fail(f"{who}: ids must be an integer tensor, got dtype {ids.dtype}")
@@ -556,8 +558,8 @@ def embedding_gather(ids, indices, lut, N: int, K: int, bitwidth: int, group_siz
     if N2 != int(N):
         _fail(f"{who}: blob holds N={N2}, not {N}")
     flat = ids.reshape(-1).long().contiguous()
-    if flat.numel() and (int(flat.min()) < 0 or int(flat.max()) >= N2):
-        _fail(f"{who}: ids must lie in [0, {N2}) (got min {int(flat.min())}, max {int(flat.max())})")
+    if check_ids and flat.numel() and bool(((flat < 0) | (flat >= N2)).any()):
+        _fail(f"{who}: ids must lie in [0, {N2})")
     with _on_device_of(A):
         out = torch.empty((flat.numel(), int(K)), dtype=lut.dtype, device=lut.device)
         check(lib.flute_embedding(ctypes.byref(w), flat.data_ptr(), flat.numel(), out.data_ptr(),

@@ -265,19 +265,28 @@ class PalettizedLinear(nn.Module):
         return dict(indices2=self.indices2 if self.has_stream2 else None,
                     lut2=self.lut2 if self.has_stream2 else None, bitwidth2=b2), b2
 
-    def _fusable(self, x, max_rank):
-        """(resB, resA, bias) the fused kernels can take, or None when an operand
-        breaks their contract (dtype follows the activations)."""
-        def ok(t):
-            return t is not None and t.is_contiguous() and t.dtype == x.dtype
+    def _cast_on(self, key: str, t: torch.Tensor, device, dtype) -> torch.Tensor:
+        """t on `device` in `dtype`, contiguous; converted once and kept (artifact readers
+        hand over float16 residual factors whatever the activation dtype is)."""
+        k = (key, str(device), str(dtype), t.data_ptr())
+        if k not in self._dev_cache:
+            self._dev_cache[k] = t.detach().to(device=device, dtype=dtype).contiguous()
+        return self._dev_cache[k]
+
+    def _fusable(self, x, max_rank, device=None):
+        """(resB, resA, bias) the fused kernels can take: in the activation dtype, contiguous,
+        on the device of x; None when the rank is beyond the kernels' limit.  Operands in
+        another floating dtype are converted once per (device, dtype) and cached."""
+        device = x.device if device is None else device
         resB = resA = None
         if self.has_residual():
-            if not (ok(self.resA) and ok(self.resB)) or self.resB.shape[0] > max_rank:
+            if self.resB.shape[0] > max_rank:
                 return None
-            resB, resA = self.resB, self.resA
+            resB = self._cast_on("resB", self.resB, device, x.dtype)
+            resA = self._cast_on("resA", self.resA, device, x.dtype)
         bias = self.bias
-        if bias is not None and not ok(bias):
-            return None
+        if bias is not None:
+            bias = self._cast_on("bias", bias, device, x.dtype)
         return resB, resA, bias
 
     def _gemv_route(self, x, rotated_in_kernel: bool):
@@ -290,6 +299,8 @@ class PalettizedLinear(nn.Module):
             return None
         if self.lut.dtype not in (torch.float16, torch.bfloat16):
             return None
+        if self.lut.dtype == torch.bfloat16 and x.dtype != torch.bfloat16:
+            return None                     # the kernels refuse this pair: a routing decision here
         kw, b2 = self._stream_kwargs()
         rot = {}
         if rotated_in_kernel:
@@ -381,6 +392,36 @@ class PalettizedLinear(nn.Module):
         return y.reshape(*shape[:-1], self.N)
 
 
+def _operand_problem(m, device) -> Optional[str]:
+    """Why a member's blobs and LUTs cannot be handed to a kernel by address, or None
+    (upstream's _build_state makes the same checks, :1740-1790): uint8 blobs, LUTs of
+    one 16-bit dtype, all contiguous, all on the device of the activations."""
+    def bad(t, dtype):
+        return t is None or not t.is_cuda or t.device != device or not t.is_contiguous() \
+            or t.dtype != dtype
+    if bad(m.indices, torch.uint8):
+        return "indices are not a contiguous uint8 tensor on the input's device"
+    if bad(m.lut, m.lut.dtype) or m.lut.dtype not in (torch.float16, torch.bfloat16):
+        return "lut is not a contiguous 16-bit tensor on the input's device"
+    if m.has_stream2:
+        if bad(m.indices2, torch.uint8):
+            return "stream-2 indices are not a contiguous uint8 tensor on the input's device"
+        if bad(m.lut2, m.lut.dtype):
+            return "stream-2 lut does not match the first lut's dtype and device"
+    return None
+
+
+def _operand_ptrs(members) -> tuple:
+    """Addresses a cached segment table was built from: a table is stale once any of them
+    changes (a module moved to another device and back, a buffer replaced)."""
+    out = []
+    for m in members:
+        for t in (m.indices, m.lut, getattr(m, "indices2", None), getattr(m, "lut2", None),
+                  getattr(m, "resA", None), getattr(m, "resB", None), getattr(m, "bias", None)):
+            out.append(0 if t is None else t.data_ptr())
+    return tuple(out)
+
+
 class FusedPalettizedMLP(nn.Module):
     """down(act(gate(x)) * up(x)) with the decode shape (one token) collapsed
     into one merged gate+up+SiLU*mul launch followed by the down GEMV
@@ -408,11 +449,12 @@ class FusedPalettizedMLP(nn.Module):
                 return None
             lead = (x.shape[0], x.shape[1])
             x = x.reshape(1, x.shape[2])
-        if x.dim() != 2 or x.shape[0] != 1 or not x.is_contiguous() or x.requires_grad \
-                or x.dtype not in (torch.float16, torch.bfloat16):
+        if x.dim() != 2 or x.shape[0] != 1 or not x.is_cuda or not x.is_contiguous() \
+                or x.requires_grad or x.dtype not in (torch.float16, torch.bfloat16):
             return None
         state = self._merge_state
-        if state is None or state["device"] != x.device or state["dtype"] != x.dtype:
+        if state is None or state["device"] != x.device or state["dtype"] != x.dtype or \
+                state.get("ptrs") != _operand_ptrs((self.gate_proj, self.up_proj)):
             state = self._merge_state = self._build_state(x.device, x.dtype)
         if not state["ok"]:
             return None
@@ -427,6 +469,8 @@ class FusedPalettizedMLP(nn.Module):
         (device, dtype).  `reason` says why a pair is not fused."""
         g, u = self.gate_proj, self.up_proj
         state = {"ok": False, "device": device, "dtype": dtype}
+        if isinstance(g, PalettizedLinear) and isinstance(u, PalettizedLinear):
+            state["ptrs"] = _operand_ptrs((g, u))
 
         def refuse(why):
             state["reason"] = why
@@ -444,10 +488,16 @@ class FusedPalettizedMLP(nn.Module):
             return refuse("mixed rotation presence")
         if g.lut.dtype != u.lut.dtype or g.lut.dtype not in (torch.float16, torch.bfloat16):
             return refuse("lut dtype")
+        if g.lut.dtype == torch.bfloat16 and dtype != torch.bfloat16:
+            return refuse("bfloat16 lut needs bfloat16 activations")
         fx = _flute()
         rows, keep, specs, ranks = [], [], [], []
         for m in (g, u):
-            fused = m._fusable(torch.empty(0, dtype=dtype), fx.GEMV_SPLITK_MAX_RESIDUAL_RANK)
+            why = _operand_problem(m, device)
+            if why is not None:
+                return refuse(why)
+            fused = m._fusable(torch.empty(0, dtype=dtype), fx.GEMV_SPLITK_MAX_RESIDUAL_RANK,
+                               device=device)
             if fused is None:
                 return refuse("residual/bias contract")
             resB, resA, bias = fused
@@ -463,7 +513,7 @@ class FusedPalettizedMLP(nn.Module):
                          ptr(m.lut2) if b2 else 0, ptr(resB), ptr(resA), ptr(bias), 0, m.N,
                          0 if resB is None else int(resB.shape[0]), m.bitwidth, b2,
                          m.group_size, ptr(signs), ptr(awq)])
-            keep.append((signs, awq))
+            keep.append((signs, awq, resB, resA, bias))
             specs.append((m.bitwidth, b2, m.group_size))
             ranks.append(0 if resB is None else int(resB.shape[0]))
         if not fx.gemv_mlp_supported(g.K, g.N, specs, ranks[0], ranks[1],
@@ -507,7 +557,8 @@ class SplitQKV(nn.Module):
                 or x.requires_grad or x.dtype not in (torch.float16, torch.bfloat16):
             return None
         state = self._merge_state
-        if state is None or state["device"] != x.device or state["dtype"] != x.dtype:
+        if state is None or state["device"] != x.device or state["dtype"] != x.dtype or \
+                state.get("ptrs") != _operand_ptrs((self.q_proj, self.k_proj, self.v_proj)):
             state = self._merge_state = self._build_state(x.device, x.dtype)
         if not state["ok"]:
             return None
@@ -519,6 +570,8 @@ class SplitQKV(nn.Module):
     def _build_state(self, device, dtype):
         members = (self.q_proj, self.k_proj, self.v_proj)
         state = {"ok": False, "device": device, "dtype": dtype}
+        if all(isinstance(m, PalettizedLinear) for m in members):
+            state["ptrs"] = _operand_ptrs(members)
 
         def refuse(why):
             state["reason"] = why
@@ -533,16 +586,23 @@ class SplitQKV(nn.Module):
         if len({m.lut.dtype for m in members}) != 1 or \
                 members[0].lut.dtype not in (torch.float16, torch.bfloat16):
             return refuse("lut dtype")
+        if members[0].lut.dtype == torch.bfloat16 and dtype != torch.bfloat16:
+            return refuse("bfloat16 lut needs bfloat16 activations")
         rot = [m.rot_signs is not None for m in members]
         if any(rot) and not all(rot):
             return refuse("mixed rotation presence")
+        for m in members:
+            why = _operand_problem(m, device)
+            if why is not None:
+                return refuse(why)
         fx = _flute()
         total = sum(m.N for m in members)
         out = torch.zeros(1, total, dtype=dtype, device=device)
         rows, keep, specs, off = [], [], [], 0
         esize = out.element_size()
         for m in members:
-            fused = m._fusable(torch.empty(0, dtype=dtype), fx.GEMV_SPLITK_MAX_RESIDUAL_RANK)
+            fused = m._fusable(torch.empty(0, dtype=dtype), fx.GEMV_SPLITK_MAX_RESIDUAL_RANK,
+                               device=device)
             if fused is None:
                 return refuse("residual/bias contract")
             resB, resA, bias = fused
@@ -555,6 +615,7 @@ class SplitQKV(nn.Module):
             b2 = m.bitwidth2 if m.has_stream2 else 0
             ptr = lambda t: 0 if t is None else t.data_ptr()
             rank = 0 if resB is None else int(resB.shape[0])
+            keep.append((resB, resA, bias))
             rows.append([ptr(m.indices), ptr(m.lut), ptr(m.indices2) if b2 else 0,
                          ptr(m.lut2) if b2 else 0, ptr(resB), ptr(resA), ptr(bias),
                          out.data_ptr() + off * esize, m.N, rank, m.bitwidth, b2, m.group_size,
@@ -663,7 +724,10 @@ class PalettizedEmbedding(nn.Module):
             raise ValueError(f"PalettizedEmbedding.forward: ids must be an integer tensor, got "
                              f"dtype {ids.dtype}")
         ids = ids.long()
-        if ids.numel() and (int(ids.min()) < 0 or int(ids.max()) >= self.N):
+        capturing = ids.is_cuda and torch.cuda.is_current_stream_capturing()
+        # one reduction and one host read; skipped under graph capture, where no value can
+        # reach the host (the kernel writes a row of zeros for an id outside the table)
+        if ids.numel() and not capturing and bool(((ids < 0) | (ids >= self.N)).any()):
             raise ValueError(f"PalettizedEmbedding.forward: ids must lie in [0, {self.N})")
         if not self.reference and ids.is_cuda:
             _count("embedding_gather")
@@ -672,7 +736,7 @@ class PalettizedEmbedding(nn.Module):
                 ids, self.indices, self.lut, self.N, self.K, self.bitwidth, self.group_size,
                 indices2=self.indices2, lut2=self.lut2,
                 bitwidth2=self.bitwidth2 if self.has_stream2 else 0,
-                resB=self.resB, resA=self.resA, signs=signs)
+                resB=self.resB, resA=self.resA, signs=signs, check_ids=False)
         w = self._gather_stream(ids, self.lut, 1)
         if self.has_stream2:
             w = w + self._gather_stream(ids, self.lut2, 2)

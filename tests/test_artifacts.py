@@ -144,3 +144,37 @@ def test_qkv_components(tmp_path):
     assert rel_l2(m(x), ref) <= 1e-3
     with pytest.raises(ValueError, match="bias length"):
         artifacts.load_palettized_weight(meta, tmp, bias=torch.zeros(500).half(), reference=True)
+
+
+@pytest.mark.parametrize("where,order,compensated", [
+    ("awq", "rotate_then_awq", True),          # the record's own awq.fold_order
+    ("awq", "awq_then_rotate", False),
+    ("rotation", "awq_then_rotate", False),    # only rotation.order records it
+    ("rotation", "rotate_then_awq", True),
+    (None, None, True),                        # no record: the legacy rotate-then-AWQ order
+])
+def test_awq_scale_map_with_tensor_values(tmp_path, where, order, compensated):
+    """The scale map holds (K,) tensors (a truth test on one is an error), the fold order
+    comes from awq.fold_order, else rotation.order, and decides whether the compensated
+    rotation ((x * s) @ T) / s or the plain one runs."""
+    w = make_weight(256, 128, bits=4, gs=128, seed=11)
+    meta = _write(str(tmp_path), "layers_0_mlp_down_proj", w)
+    meta["rotation"] = {"seed": 7, "k": 128}
+    if where == "awq":
+        meta["awq"] = {"fold_order": order}
+    elif where == "rotation":
+        meta["rotation"]["order"] = order
+    s = torch.rand(128, generator=torch.Generator().manual_seed(3)) + 0.5
+    scales = {"layers_0_mlp_down_proj": s, "someone_else": torch.ones(128)}
+    m = artifacts.load_palettized_weight(meta, str(tmp_path), reference=True, awq_scales=scales)
+    assert m.awq_scale is not None and torch.equal(m.awq_scale, s)
+    assert m.fold_order == (order or "rotate_then_awq")
+    assert m._compensated() is compensated
+    x = make_x(2, 128, seed=5)
+    signs = O.rotation_signs(128, 7)
+    xr = O.fht_awq_reference(x, signs, s) if compensated else O.fht_reference(x, signs)
+    assert rel_l2(m(x), _exact(w, xr).half()) <= 2e-3
+    # a tensor the map does not name stays unscaled
+    m0 = artifacts.load_palettized_weight(meta, str(tmp_path), reference=True,
+                                          awq_scales={"other": s})
+    assert m0.awq_scale is None

@@ -302,3 +302,32 @@ def test_tuning_is_read_once_and_on_reload(monkeypatch):
         monkeypatch.undo()
         _lib.lib.flute_reload_tuning()
     assert before(w, 1) == base
+
+
+def test_merged_modules_refuse_operands_they_cannot_pass_by_address():
+    """The merged launches read raw addresses out of a table: members left on the CPU, a
+    stream-2 LUT of another dtype, or a non-contiguous blob must end in the per-module chain
+    (a refusal with a reason), never in a kernel launch."""
+    wg, wu = make_weight(256, 128, seed=1, bits2=2), make_weight(256, 128, seed=2, bits2=2)
+
+    def member(w, **over):
+        args = dict(indices2=w["blob2"], lut2=w["lut2"], bitwidth2=2, reference=False)
+        args.update(over)
+        return pm.PalettizedLinear(w["blob"], w["lut"], 4, 128, 256, 128, **args)
+
+    silu = torch.nn.functional.silu
+    cpu = torch.device("cpu")
+    mlp = pm.FusedPalettizedMLP(member(wg), member(wu), member(wg), silu)
+    assert "device" in mlp._build_state(cpu, torch.float16)["reason"]      # CPU members
+    assert mlp._fused_gate_up(make_x(1, 128)) is None                      # and a CPU input
+    qkv = pm.SplitQKV(member(wg), member(wu), member(wg))
+    assert "device" in qkv._build_state(cpu, torch.float16)["reason"]
+    # the verdict names the first problem it meets; each is a refusal of its own
+    m = member(wg)
+    assert "indices" in pm._operand_problem(m, cpu)
+    m.lut2 = m.lut2.float()
+    assert pm._operand_problem(m, cpu) is not None
+    # pointer tuple: replacing a buffer changes it, so a cached table would be rebuilt
+    before = pm._operand_ptrs((m,))
+    m.indices = m.indices.clone()
+    assert pm._operand_ptrs((m,)) != before

@@ -154,6 +154,34 @@ def test_fused_mlp_module():
     assert rel_l2(y.cpu(), mref(x)) <= 2e-3       # two 16-bit roundings (h, then y) on each side
 
 
+def test_merged_tables_follow_moved_and_converted_members():
+    """The cached segment table holds raw addresses.  A member moved to the CPU and back has
+    new buffers: the table is rebuilt (stale addresses would be a memory fault).  Residual
+    factors kept in float16 are converted once for bfloat16 activations, so the merged
+    launch still serves them."""
+    H, I = 512, 1024
+    wg, wu, wd = (make_weight(I, H, seed=1, rank=8), make_weight(I, H, seed=2, rank=8),
+                  make_weight(H, I, seed=3))
+    refs, kers = zip(*[_modules(w) for w in (wg, wu, wd)])
+    act = torch.nn.functional.silu
+    mref, mker = pm.FusedPalettizedMLP(*refs, act), pm.FusedPalettizedMLP(*kers, act)
+    x = make_x(1, H, seed=7)
+    y0 = mker(x.to(DEV))
+    first = mker._merge_state
+    assert first["ok"]
+    mker.gate_proj.to("cpu")
+    mker.gate_proj.to(DEV)
+    y1 = mker(x.to(DEV))
+    assert mker._merge_state is not first and mker._merge_state["ok"]
+    assert torch.equal(y0, y1)
+    # bfloat16 activations against float16 residual factors: merged launch, not the fallback
+    xb = make_x(1, H, seed=8, dtype=torch.bfloat16)
+    pm.ROUTE_CENSUS.clear()
+    yb = mker(xb.to(DEV))
+    assert pm.ROUTE_CENSUS.get("gemv_mlp") == 1
+    assert rel_l2(yb.cpu(), mref(xb)) <= 8e-3     # bf16 h and y, residual factors rounded to bf16
+
+
 def test_fused_mlp_module_replays_from_a_graph():
     """The module layer is host-bound in eager mode (tens of microseconds of Python per
     call against ~20 us of kernels), so decode loops capture it in a HIP graph.  Every
