@@ -214,6 +214,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const bool x_direct = staged_signs == nullptr;  // plain copy
     const bool x_short = kc <= XV * NT * 8;         // uniform
     uint4 q[PF];
+    // bfloat16 activations in front of a float16 LUT: the staged row is x * 2^-xshift
+    const bool convert = !BF16 && p.act_bf16;       // uniform
+    uint32_t *slots = (uint32_t *)red;
+    int xshift = 0;
     if (x_direct && x_short) {
         // The usual case: activations first, then two index loads, the table (its LUT
         // row arrives through the scalar cache meanwhile), the rest of the loads, and
@@ -232,10 +236,19 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         }
         write_table(lrow);
         first_units(qrow, q, PF0);
+        if (convert) {
+            uint32_t e = 0;
+#pragma unroll
+            for (int i = 0; i < XV; ++i)
+                if ((i * NT + tid) * 8 < kc) e = max(e, bf16_max_exp8(xv[i]));
+            xshift = bf16_row_shift(workgroup_max(e, slots, tid, NT));
+#pragma unroll
+            for (int i = 0; i < XV; ++i) xv[i] = bf16_to_f16_scaled8(xv[i], xshift);
+        }
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
             const int j = (i * NT + tid) * 8;
-            if (j < kc) stage8(j, to_compute_type<BF16>(xv[i], p.act_bf16));
+            if (j < kc) stage8(j, xv[i]);
         }
     } else if (x_direct) {
         // A long K range: the index registers carry the activations first.
@@ -245,13 +258,24 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             q[n] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
         }
         __builtin_amdgcn_sched_barrier(0);
+        if (convert) {
+            uint32_t e = 0;
+#pragma unroll
+            for (int n = 0; n < PF; ++n)
+                if ((n * NT + tid) * 8 < kc) e = max(e, bf16_max_exp8(q[n]));
+            for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8)
+                e = max(e, bf16_max_exp8(*(const uint4 *)(staged_x + k0 + j)));
+            xshift = bf16_row_shift(workgroup_max(e, slots, tid, NT));
+        }
 #pragma unroll
         for (int n = 0; n < PF; ++n) {
             const int j = (n * NT + tid) * 8;
-            if (j < kc) stage8(j, to_compute_type<BF16>(q[n], p.act_bf16));
+            if (j < kc) stage8(j, convert ? bf16_to_f16_scaled8(q[n], xshift) : q[n]);
         }
-        for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8)
-            stage8(j, to_compute_type<BF16>(*(const uint4 *)(staged_x + k0 + j), p.act_bf16));
+        for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8) {
+            const uint4 v = *(const uint4 *)(staged_x + k0 + j);
+            stage8(j, convert ? bf16_to_f16_scaled8(v, xshift) : v);
+        }
         write_table(lrow);
         __builtin_amdgcn_sched_barrier(0);
         first_units(qrow, q, 0);
@@ -263,7 +287,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             q[n] = load_idx16(qrow + (size_t)n * step + lane0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
+        xshift = stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
         write_table(lrow);
         __builtin_amdgcn_sched_barrier(0);
         first_units(qrow, q, PF0);
@@ -420,7 +444,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 #pragma unroll
                 for (int gb = 0; gb < GPI; ++gb)
                     y += red[(so * NW + ww) * 32 + ((gb << SH) | cgl_o) * 8 + a_o];
-            yv[so] = y;
+            yv[so] = ldexpf(y, xshift);             // undo the activation scaling (exact)
         }
     }
 

@@ -288,18 +288,71 @@ __device__ __forceinline__ void load_act8(const uint16_t *x, int k, int is_bf16,
     }
 }
 
-// Eight raw activations -> eight values of the compute type.
-template <bool BF16>
-__device__ __forceinline__ uint4 to_compute_type(uint4 v, int act_bf16) {
-    if (act_bf16 && !BF16) {                       // bf16 activations, fp16 compute type
-        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+// ---- bfloat16 activations in front of float16 arithmetic -------------------------
+// A float16 LUT fixes the arithmetic type to float16 (the dequantised weight must be the
+// LUT entry exactly), but bfloat16 activations reach from 1e-38 to 3e38 and float16 only
+// from 6e-8 to 65504.  The staged row is therefore scaled by a power of two chosen from
+// its largest magnitude (exact: only the exponent changes), the products are summed in
+// fp32 as usual, and the row sums are scaled back before anything else is added.  The
+// result is what unscaled arithmetic would give wherever that does not overflow, and
+// stays finite and correct where it would.
+
+// Largest biased exponent among eight bfloat16 values.
+__device__ __forceinline__ uint32_t bf16_max_exp8(uint4 v) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t e = 0;
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-            w[q] = (uint32_t)f2h(bf2f((uint16_t)(w[q] & 0xffffu))) |
-                   ((uint32_t)f2h(bf2f((uint16_t)(w[q] >> 16))) << 16);
-        v = make_uint4(w[0], w[1], w[2], w[3]);
+    for (int q = 0; q < 4; ++q) {
+        e = max(e, (w[q] >> 7) & 0xffu);
+        e = max(e, (w[q] >> 23) & 0xffu);
     }
-    return v;
+    return e;
+}
+
+// Maximum over the workgroup; slots = one LDS word per wavefront.  One barrier.
+__device__ __forceinline__ uint32_t workgroup_max(uint32_t v, uint32_t *slots, int tid,
+                                                  int nthreads) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) v = max(v, (uint32_t)__shfl_xor((int)v, m));
+    if ((tid & 63) == 0) slots[tid >> 6] = v;
+    __syncthreads();
+    uint32_t r = 0;
+    for (int w = 0; w < (nthreads >> 6); ++w) r = max(r, slots[w]);
+    return r;
+}
+
+// Shift that brings a row whose largest biased exponent is emax to magnitudes in [1, 2):
+// the largest value then has 15 binades of float16 range above it and 14 normal (24 in
+// all) below.  Zero rows and non-finite values keep their values (shift 0).
+__device__ __forceinline__ int bf16_row_shift(uint32_t emax) {
+    return (emax == 0 || emax == 255) ? 0 : (int)emax - 127;
+}
+
+// Eight bfloat16 values -> eight float16 values of x * 2^-shift.
+__device__ __forceinline__ uint4 bf16_to_f16_scaled8(uint4 v, int shift) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float lo = ldexpf(bf2f((uint16_t)(w[q] & 0xffffu)), -shift);
+        const float hi = ldexpf(bf2f((uint16_t)(w[q] >> 16)), -shift);
+        w[q] = (uint32_t)f2h(lo) | ((uint32_t)f2h(hi) << 16);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// xs holds kc bfloat16 values in natural order, written by every thread of the
+// workgroup; converts them in place to float16 of x * 2^-shift and returns the shift.
+// Barriers inside: before (the writes), between, and none after (the caller's next
+// barrier publishes the result).
+__device__ __forceinline__ int normalise_staged_row(uint16_t *xs, int kc, uint32_t *slots, int tid,
+                                                    int nthreads) {
+    __syncthreads();
+    uint32_t e = 0;
+    for (int j = tid * 8; j < kc; j += nthreads * 8) e = max(e, bf16_max_exp8(*(const uint4 *)(xs + j)));
+    const int shift = bf16_row_shift(workgroup_max(e, slots, tid, nthreads));
+    for (int j = tid * 8; j < kc; j += nthreads * 8)
+        *(uint4 *)(xs + j) = bf16_to_f16_scaled8(*(const uint4 *)(xs + j), shift);
+    return shift;
 }
 
 // Output side of the fused rotation, eight columns per step: value * sign * inv
@@ -320,8 +373,7 @@ __device__ __forceinline__ void rotated_out8(const float *buf, int j, const floa
         float t = buf[s0 ^ q] * sg[q] * inv;
         if (awq) t = t / sc[q];
         const uint16_t a = round_act(t, act_bf16);
-        const float back = act_bf16 ? bf2f(a) : h2f(a);
-        const uint32_t h = BF16 ? f2bf(back) : f2h(back);
+        const uint32_t h = a;       // the activation type; the caller converts bf16 -> f16 if needed
         if (q & 1) o[q >> 1] |= h << 16;
         else o[q >> 1] = h;
     }
@@ -420,8 +472,7 @@ __device__ __forceinline__ void rotate_blocks_inwave(const uint16_t *x, const fl
                 float t = f[h][q] * sg[h][q] * inv;
                 if (awq) t = t / sc[h][q];
                 const uint16_t a = round_act(t, act_bf16);
-                const float back = act_bf16 ? bf2f(a) : h2f(a);
-                const uint32_t v = BF16 ? f2bf(back) : f2h(back);
+                const uint32_t v = a;   // the activation type; the caller converts bf16 -> f16 if needed
                 if (q & 1) o[q >> 1] |= v << 16;
                 else o[q >> 1] = v;
             }
@@ -543,8 +594,7 @@ __device__ __forceinline__ void rotate_segment_fast(const uint16_t *x, const flo
                 float t = f[h][q] * sg[h][q] * inv;
                 if (awq) t = t / sc[h][q];
                 const uint16_t a = round_act(t, act_bf16);
-                const float back = act_bf16 ? bf2f(a) : h2f(a);
-                const uint32_t v = BF16 ? f2bf(back) : f2h(back);
+                const uint32_t v = a;   // the activation type; the caller converts bf16 -> f16 if needed
                 if (q & 1) o[q >> 1] |= v << 16;
                 else o[q >> 1] = v;
             }
@@ -559,22 +609,30 @@ __device__ __forceinline__ void rotate_segment_fast(const uint16_t *x, const flo
 // that overlaps the slice is computed first in the fp32 scratch at the start of
 // LDS (where the tables are built afterwards), rounded to the activation type
 // exactly as the standalone rotation kernel rounds, and only then converted.
+// bfloat16 activations in front of a float16 LUT are scaled by a power of two on the
+// way (normalise_staged_row); the shift is returned and is 0 otherwise.
 // Ends with the slice complete and the scratch free (barrier included).
 template <bool BF16>
-__device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *signs,
-                        const float *awq, uint8_t *lds, int k0, int kc, int tid, int nthreads) {
+__device__ int stage_x(const GemvParams &p, const uint16_t *x, const float *signs,
+                       const float *awq, uint8_t *lds, int k0, int kc, int tid, int nthreads) {
     uint16_t *xs = (uint16_t *)(lds + p.lds_x);
+    const bool convert = !BF16 && p.act_bf16;          // uniform
+    auto finish = [&]() -> int {
+        int shift = 0;
+        if (convert)
+            shift = normalise_staged_row(xs, kc, (uint32_t *)(lds + p.lds_red), tid, nthreads);
+        __syncthreads();
+        return shift;
+    };
     if (signs == nullptr) {
         for (int j = tid * 8; j < kc; j += nthreads * 8)
-            *(uint4 *)(xs + j) = to_compute_type<BF16>(*(const uint4 *)(x + k0 + j), p.act_bf16);
-        __syncthreads();
-        return;
+            *(uint4 *)(xs + j) = *(const uint4 *)(x + k0 + j);
+        return finish();
     }
     float *buf = (float *)lds;
     if (p.fht_block > 0 && p.fht_block <= 256) {
         rotate_blocks_inwave<BF16>(x, signs, awq, xs, k0, kc, p.fht_block, p.act_bf16, tid, nthreads);
-        __syncthreads();
-        return;
+        return finish();
     }
     if (p.fht_block > 0) {
         // equal blocks: the slice is a whole number of blocks
@@ -588,8 +646,7 @@ __device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *sig
 #pragma unroll 2
         for (int j = tid * 8; j < kc; j += nthreads * 8)
             rotated_out8<BF16>(buf, j, signs, awq, k0 + j, inv, p.act_bf16, xs + j);
-        __syncthreads();
-        return;
+        return finish();
     }
     // descending power-of-two segments of K (fht.py:118-134 upstream)
     for (int off = 0, rem = p.K; rem > 0;) {
@@ -617,6 +674,7 @@ __device__ void stage_x(const GemvParams &p, const uint16_t *x, const float *sig
         off += b;
         rem -= b;
     }
+    return finish();
 }
 
 // Geometry of this lane inside its workgroup, fixed for the whole kernel.
@@ -941,7 +999,10 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     constexpr int XV = 2;                           // 16-byte activation loads per thread
     StreamRegs<BF> first;
     const uint16_t *x0 = sg.xsrc ? sg.xsrc : p.x;
-    const bool x_ahead = BFIX != 0 && sg.signs == nullptr;      // uniform
+    // bfloat16 activations with a float16 LUT are scaled on the way into LDS: that needs
+    // the whole slice first, so such launches stage through stage_x
+    const bool x_ahead = BFIX != 0 && sg.signs == nullptr && !(!BF16 && p.act_bf16);   // uniform
+    int xshift = 0;                                 // the staged slice holds x * 2^-xshift
     if (x_ahead) {
         uint4 xv[XV];
 #pragma unroll
@@ -954,15 +1015,16 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
             const int j = (i * gm.nthreads + gm.tid) * 8;
-            if (j < kc) *(uint4 *)(xs + j) = to_compute_type<BF16>(xv[i], p.act_bf16);
+            if (j < kc) *(uint4 *)(xs + j) = xv[i];
         }
         for (int j = (XV * gm.nthreads + gm.tid) * 8; j < kc; j += gm.nthreads * 8)
-            *(uint4 *)(xs + j) = to_compute_type<BF16>(*(const uint4 *)(x0 + k0 + j), p.act_bf16);
+            *(uint4 *)(xs + j) = *(const uint4 *)(x0 + k0 + j);
         // no barrier here: the one after the table build publishes both
     } else {
-        stage_x<BF16>(p, x0, sg.signs, sg.awq, lds, k0, kc, gm.tid, gm.nthreads);
+        xshift = stage_x<BF16>(p, x0, sg.signs, sg.awq, lds, k0, kc, gm.tid, gm.nthreads);
         if constexpr (BFIX != 0) stream_issue<BF>(p, sg, sg.st[0], gm, first);
     }
+    int out_shift[2] = {0, 0};
     const uint16_t *staged_x = x0;
     const float *staged_signs = sg.signs, *staged_awq = sg.awq;
 
@@ -970,11 +1032,12 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
         const GemvSeg og = kp->seg[so == 1 ? 1 : si0];
         const uint16_t *xin = og.xsrc ? og.xsrc : p.x;
         if (so > 0 && (xin != staged_x || og.signs != staged_signs || og.awq != staged_awq)) {
-            stage_x<BF16>(p, xin, og.signs, og.awq, lds, k0, kc, gm.tid, gm.nthreads);
+            xshift = stage_x<BF16>(p, xin, og.signs, og.awq, lds, k0, kc, gm.tid, gm.nthreads);
             staged_x = xin;
             staged_signs = og.signs;
             staged_awq = og.awq;
         }
+        out_shift[so] = xshift;
         float acc[8];
 #pragma unroll
         for (int a = 0; a < 8; ++a) acc[a] = 0.0f;
@@ -1021,7 +1084,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
             if (so >= nout) break;
             float y = 0.0f;
             for (int w = 0; w < gm.nwaves; ++w) y += red[(so * gm.nwaves + w) * 32 + gm.tid];
-            yv[so] = y;
+            yv[so] = ldexpf(y, out_shift[so]);      // undo the activation scaling (exact)
         }
     }
 

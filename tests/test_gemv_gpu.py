@@ -247,3 +247,55 @@ def test_workspace_growth_is_refused_under_graph_capture():
     g2.replay()
     torch.cuda.synchronize()
     assert torch.equal(y, want)
+
+
+def _wide_range_row(K, kind):
+    """bfloat16 activations that float16 cannot hold: a few values near 1e5 among N(0, 1)
+    ones, a whole row around 1e-7, a whole row around 1e30, and a row mixing 1e5 with 1e-6."""
+    x = make_x(1, K, seed=19, dtype=torch.float32)
+    if kind == "outliers":
+        x[0, [3, K // 2, K - 1]] = torch.tensor([1.0e5, -2.5e5, 9.0e4])
+    elif kind == "tiny":
+        x *= 1.0e-7
+    elif kind == "huge":
+        x *= 1.0e30
+    else:
+        x[0, ::2] *= 1.0e-6
+        x[0, 1::64] *= 1.0e5
+    return x.to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("kind", ["outliers", "tiny", "huge", "mixed"])
+@pytest.mark.parametrize("bits,split,rot", [(4, 0, False), (4, 4, False), (3, 0, False),
+                                            (4, 0, True), (2, 2, True)])
+def test_bf16_activations_beyond_the_float16_range(kind, bits, split, rot):
+    """A float16 LUT makes the kernels multiply in float16; bfloat16 activations outside
+    float16's range (|x| > 65504, |x| < 6e-8) must still give the reference forward's
+    result (x.float() @ W.t(), scripts/palettized_modules.py:1241-1251), never inf or 0."""
+    N, K = 512, 4096
+    w = make_weight(N, K, bits, 128, seed=23 + bits, act_dtype=torch.bfloat16, device=DEV)
+    x = _wide_range_row(K, kind)
+    signs = O.rotation_signs(K, 4) if rot else None
+    y = _run(w, x, signs=signs, split=split).cpu()
+    assert y.dtype == torch.bfloat16 and torch.isfinite(y).all()
+    ref = O.linear_reference(x, w["blob"].numpy(), w["lut"], N, K, 128, bits, signs=signs)
+    assert torch.isfinite(ref).all() and ref.abs().max() > 0
+    assert rel_l2(y, ref) <= TOL
+
+
+def test_merged_gate_up_with_activations_beyond_the_float16_range():
+    N, K = 1024, 4096
+    g = make_weight(N, K, 4, 128, seed=27, act_dtype=torch.bfloat16, device=DEV)
+    u = make_weight(N, K, 4, 128, seed=28, act_dtype=torch.bfloat16, device=DEV)
+    x = _wide_range_row(K, "outliers")
+    table = torch.tensor([[g["blob_d"].data_ptr(), g["lut_d"].data_ptr(), 0, 0, 0, 0, 0, 0, N, 0, 4, 0,
+                           128, 0, 0],
+                          [u["blob_d"].data_ptr(), u["lut_d"].data_ptr(), 0, 0, 0, 0, 0, 0, N, 0, 4, 0,
+                           128, 0, 0]], dtype=torch.int64)
+    out = torch.zeros(1, N, dtype=torch.bfloat16, device=DEV)
+    fx.qgemm_gemv_mlp(x.to(DEV), table, out)
+    yg = O.linear_exact(x, g["blob"].numpy(), g["lut"], N, K, 128, 4)
+    yu = O.linear_exact(x, u["blob"].numpy(), u["lut"], N, K, 128, 4)
+    ref = O.silu_mul_exact(yg, yu).to(torch.bfloat16)
+    assert torch.isfinite(out).all()
+    assert rel_l2(out.cpu(), ref) <= 4e-3       # one bfloat16 rounding of a product of two sums
