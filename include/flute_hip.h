@@ -54,6 +54,12 @@ typedef enum flute_dtype {
  * lut1/2  [ceil(N/group_size), 2^b] in lut_dtype, contiguous
  * b2 == 0 means "single stream" and q2/lut2 are ignored
  * resB    (R, K), resA (N, R), bias (N,) in the ACTIVATION dtype, or NULL / R = 0
+ * Arithmetic type: the products run in lut_dtype, so that the dequantised weight is the
+ * LUT entry exactly.  bfloat16 activations with a float16 LUT are scaled by a power of
+ * two per staged row (exact) on their way into the kernel and the row sums are scaled
+ * back, so activations beyond float16's range (|x| > 65504, |x| < 6e-8) give the same
+ * result as fp32 arithmetic on x.float().  float16 activations with a bfloat16 LUT are
+ * refused (FLUTE_ERR_UNSUPPORTED): that conversion is not exact.
  * signs   (K,) fp32 +-1: when non-NULL the input is rotated first, x <- x @ T
  *         (fht.py:19-35); awq (K,) fp32 then selects ((x*s) @ T) / s
  */

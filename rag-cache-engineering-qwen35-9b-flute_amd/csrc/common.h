@@ -102,4 +102,72 @@ __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
     }
 }
 
+// ---- bfloat16 activations in front of float16 arithmetic -------------------------
+// A float16 LUT fixes the arithmetic type to float16 (the dequantised weight must be the
+// LUT entry exactly), but bfloat16 activations reach from 1e-38 to 3e38 and float16 only
+// from 6e-8 to 65504.  The staged row is therefore scaled by a power of two chosen from
+// its largest magnitude (exact: only the exponent changes), the products are summed in
+// fp32 as usual, and the row sums are scaled back before anything else is added.  The
+// result is what unscaled arithmetic would give wherever that does not overflow, and
+// stays finite and correct where it would.
+
+// Largest biased exponent among eight bfloat16 values.
+__device__ __forceinline__ uint32_t bf16_max_exp8(uint4 v) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t e = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        e = max(e, (w[q] >> 7) & 0xffu);
+        e = max(e, (w[q] >> 23) & 0xffu);
+    }
+    return e;
+}
+
+// Maximum over the wavefront, in scalar registers: four DPP steps fold each row of 16
+// lanes, four lane reads fold the rows.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_max(uint32_t v) {
+    const uint32_t moved = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+    return max(v, moved);
+}
+__device__ __forceinline__ uint32_t wavefront_max(uint32_t v) {
+    v = dpp_max<0xB1>(v);    // quad_perm [1,0,3,2]
+    v = dpp_max<0x4E>(v);    // quad_perm [2,3,0,1]
+    v = dpp_max<0x141>(v);   // row_half_mirror
+    v = dpp_max<0x140>(v);   // row_mirror
+    const uint32_t a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const uint32_t c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return max(max(a, b), max(c, d));
+}
+
+// Maximum over the workgroup; slots = one LDS word per wavefront.  One barrier.
+__device__ __forceinline__ uint32_t workgroup_max(uint32_t v, uint32_t *slots, int tid,
+                                                  int nthreads) {
+    v = wavefront_max(v);
+    if ((tid & 63) == 0) slots[tid >> 6] = v;
+    __syncthreads();
+    uint32_t r = 0;
+    for (int w = 0; w < (nthreads >> 6); ++w) r = max(r, slots[w]);
+    return r;
+}
+
+// Shift that brings a row whose largest biased exponent is emax to magnitudes in [1, 2):
+// the largest value then has 15 binades of float16 range above it and 14 normal (24 in
+// all) below.  Zero rows and non-finite values keep their values (shift 0).
+__device__ __forceinline__ int bf16_row_shift(uint32_t emax) {
+    return (emax == 0 || emax == 255) ? 0 : (int)emax - 127;
+}
+
+// Eight bfloat16 values -> eight float16 values of x * 2^-shift.
+__device__ __forceinline__ uint4 bf16_to_f16_scaled8(uint4 v, int shift) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const float lo = ldexpf(bf2f((uint16_t)(w[q] & 0xffffu)), -shift);
+        const float hi = ldexpf(bf2f((uint16_t)(w[q] >> 16)), -shift);
+        w[q] = (uint32_t)f2h(lo) | ((uint32_t)f2h(hi) << 16);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 }  // namespace flute

@@ -213,9 +213,12 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     const size_t xb_floats = ((size_t)M * w->R + 3) & ~(size_t)3;
     const size_t ap_floats = (size_t)p.G * 2 * p.mblk_pad * 64 * 4;
     const size_t rot_floats = w->signs ? ((size_t)M * w->K / 2 + 4) & ~(size_t)3 : 0;
+    // bfloat16 activations presented as float16 operands: one power-of-two scale per row
+    const bool scale_rows = act_dtype == FLUTE_BF16 && w->lut_dtype == FLUTE_F16;
+    const size_t shift_floats = scale_rows ? ((size_t)M + 3) & ~(size_t)3 : 0;
     float *base = nullptr;
     int *tickets = nullptr;
-    st = get_workspace(p_floats + xb_floats + ap_floats + rot_floats + 64, (size_t)units + 1, stream, &base,
+    st = get_workspace(p_floats + xb_floats + ap_floats + rot_floats + shift_floats + 64, (size_t)units + 1, stream, &base,
                        &tickets);
     if (st != FLUTE_OK) return st;
     p.P = base;
@@ -237,9 +240,22 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
             p.a_bf16 = act_dtype == FLUTE_BF16;
         }
     }
+    int *rowshift = scale_rows
+        ? (int *)(base + p_floats + xb_floats + ap_floats + rot_floats) : nullptr;
+    auto launch_rowshift = [&](const void *rows, int64_t ld) -> flute_status {
+        hipLaunchKernelGGL(gemm_rowshift_kernel, dim3(M), dim3(256), 0, stream,
+                           (const uint16_t *)rows, ld, w->K, rowshift);
+        FLUTE_HIP_CHECK(hipGetLastError());
+        p.rowshift = rowshift;
+        return FLUTE_OK;
+    };
     if (p.A8) {
-        // nothing to prepare
-    } else if (w->signs && w->R == 0) {
+        // nothing to prepare but the row scales
+        if (scale_rows) {
+            st = launch_rowshift(A, lda);
+            if (st != FLUTE_OK) return st;
+        }
+    } else if (w->signs && w->R == 0 && !scale_rows) {
         // the rotation writes the operand image itself: one launch instead of two
         FhtOperandOut image_out = {(uint32_t *)Ap, p.mblk_pad, (int)(w->lut_dtype == FLUTE_BF16)};
         st = fht_launch(A, lda, w->signs, w->awq, nullptr, 0, M, w->K, act_dtype, 0, w->rot_block,
@@ -247,8 +263,8 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
         if (st != FLUTE_OK) return st;
     } else {
         if (w->signs) {
-            // the residual coefficients need the rotated rows as rows: rotated copy first,
-            // then the ordinary pre-pass on it
+            // the residual coefficients and the row scales need the rotated rows as rows:
+            // rotated copy first, then the ordinary pre-pass on it
             void *Arot = (void *)(Ap + (size_t)p.G * 2 * p.mblk_pad * 64);
             st = fht_launch(A, lda, w->signs, w->awq, Arot, w->K, M, w->K, act_dtype, 0,
                             w->rot_block, stream, nullptr);
@@ -256,12 +272,16 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
             A = Arot;
             lda = w->K;
         }
+        if (scale_rows) {
+            st = launch_rowshift(A, lda);
+            if (st != FLUTE_OK) return st;
+        }
         const int64_t total = (int64_t)p.G * 2 * p.mblk_pad * 64;
         const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
         hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
                            (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
                            (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
-                           (int)((((uintptr_t)A & 3) == 0) && (lda % 2 == 0)));
+                           (int)((((uintptr_t)A & 3) == 0) && (lda % 2 == 0)), rowshift);
         FLUTE_HIP_CHECK(hipGetLastError());
     }
     if (w->R > 0) {

@@ -62,12 +62,14 @@ struct GemmParams {
     const u4_t *A8;        // direct mode: A itself, rows of lda8 16-byte pieces, no pre-pass
     int64_t lda8;
     int a_bf16;            // dtype of A in direct mode
+    const int *rowshift;   // [M] or NULL: row m of the operands holds A[m] * 2^-rowshift[m]
 };
 
 // Activation pre-pass: Ap[g][j][mb][lane][slot] in the LUT's 16-bit type.
 __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t *Ap, int M,
                                                         int64_t lda, int G, int mblk,
-                                                        int in_bf16, int out_bf16, int pairs) {
+                                                        int in_bf16, int out_bf16, int pairs,
+                                                        const int *rowshift) {
     const int64_t total = (int64_t)G * 2 * mblk * 64;
     for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total;
          o += (int64_t)gridDim.x * blockDim.x) {
@@ -79,6 +81,7 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t 
         const int m = mb * 16 + (lane & 15), kg = lane >> 4;
         uint32_t out[4] = {0u, 0u, 0u, 0u};
         if (m < M) {
+            const int shift = rowshift ? rowshift[m] : 0;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {              // s = ktl*2 + s2
                 const int k = g * 64 + (2 * j + (s >> 1)) * 16 + 2 * kg + 8 * (s & 1);
@@ -93,8 +96,8 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t 
                     a1 = A[m * lda + k + 1];
                 }
                 if (in_bf16 != out_bf16) {
-                    a0 = round_act(in_bf16 ? bf2f(a0) : h2f(a0), out_bf16);
-                    a1 = round_act(in_bf16 ? bf2f(a1) : h2f(a1), out_bf16);
+                    a0 = round_act(ldexpf(in_bf16 ? bf2f(a0) : h2f(a0), -shift), out_bf16);
+                    a1 = round_act(ldexpf(in_bf16 ? bf2f(a1) : h2f(a1), -shift), out_bf16);
                 }
                 out[s] = (uint32_t)a0 | ((uint32_t)a1 << 16);
             }
@@ -102,6 +105,25 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t 
         u4_t v = {out[0], out[1], out[2], out[3]};
         Ap[o] = v;
     }
+}
+
+// bfloat16 rows in front of float16 operands: shift[m] = the power of two that brings the
+// largest magnitude of row m to [1, 2) (bf16_row_shift), one workgroup per row.
+__global__ void __launch_bounds__(256) gemm_rowshift_kernel(const uint16_t *A, int64_t lda, int K,
+                                                            int *shift) {
+    __shared__ uint32_t slots[4];
+    const uint16_t *row = A + (int64_t)blockIdx.x * lda;
+    uint32_t e = 0;
+    if ((((uintptr_t)row) & 15) == 0) {                // uniform per row
+        for (int k = threadIdx.x * 8; k < K; k += 256 * 8) {
+            if (k + 8 <= K) e = max(e, bf16_max_exp8(*(const uint4 *)(row + k)));
+            else for (int q = k; q < K; ++q) e = max(e, (uint32_t)(row[q] >> 7) & 0xffu);
+        }
+    } else {
+        for (int k = threadIdx.x; k < K; k += 256) e = max(e, (uint32_t)(row[k] >> 7) & 0xffu);
+    }
+    e = workgroup_max(e, slots, threadIdx.x, 256);
+    if (threadIdx.x == 0) shift[blockIdx.x] = bf16_row_shift(e);
 }
 
 // xb[m, r] = sum_k A[m, k] * resB[r, k] in fp32 (one workgroup per (r, m)).
@@ -291,6 +313,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     const int g_first = left > 0 ? g0 : gbeg;
     const int a_row = mb0 * 16 + rho;                  // direct mode: this lane's row of A
     const bool a_row_valid = a_row < p.M;
+    const int a_shift = (DIRECT && p.rowshift && a_row_valid) ? p.rowshift[a_row] : 0;
     const u4_t *ap = DIRECT
         ? p.A8 + (int64_t)(a_row_valid ? a_row : 0) * p.lda8 + (int64_t)g_first * 8 + kg
         : p.Ap + ((int64_t)g_first * 2 * p.mblk_pad + mb0) * 64 + lane;
@@ -302,8 +325,8 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const uint16_t lo16 = (uint16_t)(raw[q] & 0xffffu), hi16 = (uint16_t)(raw[q] >> 16);
-                const float flo = p.a_bf16 ? bf2f(lo16) : h2f(lo16);
-                const float fhi = p.a_bf16 ? bf2f(hi16) : h2f(hi16);
+                const float flo = ldexpf(p.a_bf16 ? bf2f(lo16) : h2f(lo16), -a_shift);
+                const float fhi = ldexpf(p.a_bf16 ? bf2f(hi16) : h2f(hi16), -a_shift);
                 raw[q] = (uint32_t)round_act(flo, BF16) | ((uint32_t)round_act(fhi, BF16) << 16);
             }
         }
@@ -652,6 +675,11 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 y[e] = lo[e];
                 y[4 + e] = hi[e];
             }
+        }
+        if (p.rowshift) {                               // undo the row's activation scaling (exact)
+            const int sh = p.rowshift[m];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y[e] = ldexpf(y[e], sh);
         }
         if (p.R > 0) {
             const float *xr = p.xb + (size_t)m * p.R;

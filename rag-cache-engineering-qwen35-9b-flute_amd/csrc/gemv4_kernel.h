@@ -26,6 +26,11 @@
 // Per weight pair this leaves two address instructions and the lookup; the
 // multiply-accumulate and the cross-lane reduction of the dot-product form are gone.
 //
+// Activations are staged per wavefront: a wavefront loads, converts and stores exactly
+// the units of K it will read back, so the only workgroup barrier of the prologue is the
+// one that publishes the table, and a power-of-two scale (bfloat16 activations in front
+// of a float16 LUT) is a wavefront-local matter.
+//
 // The LUT row (32 bytes) comes through the scalar cache, so it does not queue
 // behind the index loads of the other workgroups of the CU in the vector memory
 // pipe; index loads are non-temporal (read once).
@@ -95,7 +100,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     constexpr int RW = LPG >> 1;                    // rows per workgroup
     constexpr int SPT = 128 / RW;                   // row slices per tile
     constexpr int SH = LPGL - 4;                    // bits of rb that pick the chunk group
-    constexpr int XV = 2;                           // 16-byte activation loads per thread
+    constexpr int XV = 4;                           // 16-byte activation loads a lane holds at once
     constexpr int PF0 = 2;                          // index loads issued ahead of the table build
     constexpr int STRIDE = 1 << ES;                 // table bytes per entry
     constexpr int CHUNKS = STRIDE / 16;             // 16-byte pieces of one entry's replicas
@@ -212,12 +217,22 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const uint16_t *staged_x = kp->seg[si0].xsrc ? kp->seg[si0].xsrc : p.x;
     const float *staged_signs = kp->seg[si0].signs, *staged_awq = kp->seg[si0].awq;
     const bool x_direct = staged_signs == nullptr;  // plain copy
-    const bool x_short = kc <= XV * NT * 8;         // uniform
     uint4 q[PF];
-    // bfloat16 activations in front of a float16 LUT: the staged row is x * 2^-xshift
+    // bfloat16 activations in front of a float16 LUT: the staged units hold x * 2^-xshift,
+    // xshift chosen per wavefront (per workgroup when the input is rotated)
     const bool convert = !BF16 && p.act_bf16;       // uniform
-    uint32_t *slots = (uint32_t *)red;
     int xshift = 0;
+    // A wavefront stages the units it consumes (unit m of wavefront w is unit w + m * NW of
+    // the K range): a 16-byte piece per lane, UPL units per wavefront load.
+    constexpr int UPL = 8 / GPI;                    // units per wavefront load
+    constexpr int LPU = 64 / UPL;                   // lanes (16-byte pieces) per unit
+    const int xu = L / LPU, xp = L % LPU;
+    auto x_piece = [&](int i) -> int {              // local k of piece i of this lane, or -1
+        const int m = i * UPL + xu;
+        return m < my_units ? (w + m * NW) * (64 * GPI) + xp * 8 : -1;
+    };
+    const int x_loads = (my_units + UPL - 1) / UPL;
+    const bool x_short = x_loads <= XV;             // uniform
     if (x_direct && x_short) {
         // The usual case: activations first, then two index loads, the table (its LUT
         // row arrives through the scalar cache meanwhile), the rest of the loads, and
@@ -225,8 +240,8 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         uint4 xv[XV];
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
-            const int j = (i * NT + tid) * 8;
-            xv[i] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
+            const int j = x_piece(i);
+            xv[i] = *(const uint4 *)(staged_x + k0 + (j >= 0 ? j : 0));
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -240,41 +255,33 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             uint32_t e = 0;
 #pragma unroll
             for (int i = 0; i < XV; ++i)
-                if ((i * NT + tid) * 8 < kc) e = max(e, bf16_max_exp8(xv[i]));
-            xshift = bf16_row_shift(workgroup_max(e, slots, tid, NT));
+                if (x_piece(i) >= 0) e = max(e, bf16_max_exp8(xv[i]));
+            xshift = bf16_row_shift(wavefront_max(e));
 #pragma unroll
             for (int i = 0; i < XV; ++i) xv[i] = bf16_to_f16_scaled8(xv[i], xshift);
         }
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
-            const int j = (i * NT + tid) * 8;
-            if (j < kc) stage8(j, xv[i]);
+            const int j = x_piece(i);
+            if (j >= 0) stage8(j, xv[i]);
         }
     } else if (x_direct) {
-        // A long K range: the index registers carry the activations first.
-#pragma unroll
-        for (int n = 0; n < PF; ++n) {
-            const int j = (n * NT + tid) * 8;
-            q[n] = *(const uint4 *)(staged_x + k0 + (j < kc ? j : 0));
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        // A long K range: two passes over this wavefront's pieces when a scale is needed
+        // (the second one reads them from the cache).
         if (convert) {
             uint32_t e = 0;
-#pragma unroll
-            for (int n = 0; n < PF; ++n)
-                if ((n * NT + tid) * 8 < kc) e = max(e, bf16_max_exp8(q[n]));
-            for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8)
-                e = max(e, bf16_max_exp8(*(const uint4 *)(staged_x + k0 + j)));
-            xshift = bf16_row_shift(workgroup_max(e, slots, tid, NT));
+            for (int i = 0; i < x_loads; ++i) {
+                const int j = x_piece(i);
+                if (j >= 0) e = max(e, bf16_max_exp8(*(const uint4 *)(staged_x + k0 + j)));
+            }
+            xshift = bf16_row_shift(wavefront_max(e));
         }
-#pragma unroll
-        for (int n = 0; n < PF; ++n) {
-            const int j = (n * NT + tid) * 8;
-            if (j < kc) stage8(j, convert ? bf16_to_f16_scaled8(q[n], xshift) : q[n]);
-        }
-        for (int j = (PF * NT + tid) * 8; j < kc; j += NT * 8) {
-            const uint4 v = *(const uint4 *)(staged_x + k0 + j);
-            stage8(j, convert ? bf16_to_f16_scaled8(v, xshift) : v);
+        for (int i = 0; i < x_loads; ++i) {
+            const int j = x_piece(i);
+            if (j >= 0) {
+                const uint4 v = *(const uint4 *)(staged_x + k0 + j);
+                stage8(j, convert ? bf16_to_f16_scaled8(v, xshift) : v);
+            }
         }
         write_table(lrow);
         __builtin_amdgcn_sched_barrier(0);
@@ -406,7 +413,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         if (!has_next) __builtin_amdgcn_s_setprio(0);
         // ---- end of an output: D[i][j] with i = (rb, kt) in (lane >> 4, register) and
         //      j = (rb', kt') in lane & 15.  The lanes with rb' == rb keep register kt';
-        //      a quad sum folds kt'. ----------------------------------------------------
+        //      a quad sum folds kt'; the activation scaling is undone here (exact). -----
         if (nso != so) {
             const bool keep = rb == kg;             // here L >> 4 is the matrix row block
 #pragma unroll
@@ -415,7 +422,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 v = keep ? v : 0.0f;
                 v = dpp_add<0xB1>(v);               // quad_perm [1,0,3,2]
                 v = dpp_add<0x4E>(v);               // quad_perm [2,3,0,1]
-                if (keep && kt == 0) red[(so * NW + w) * 32 + rb * 8 + a] = v;
+                if (keep && kt == 0) red[(so * NW + w) * 32 + rb * 8 + a] = ldexpf(v, xshift);
                 acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
@@ -444,7 +451,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 #pragma unroll
                 for (int gb = 0; gb < GPI; ++gb)
                     y += red[(so * NW + ww) * 32 + ((gb << SH) | cgl_o) * 8 + a_o];
-            yv[so] = ldexpf(y, xshift);             // undo the activation scaling (exact)
+            yv[so] = y;
         }
     }
 

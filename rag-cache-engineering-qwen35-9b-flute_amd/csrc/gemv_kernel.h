@@ -288,58 +288,6 @@ __device__ __forceinline__ void load_act8(const uint16_t *x, int k, int is_bf16,
     }
 }
 
-// ---- bfloat16 activations in front of float16 arithmetic -------------------------
-// A float16 LUT fixes the arithmetic type to float16 (the dequantised weight must be the
-// LUT entry exactly), but bfloat16 activations reach from 1e-38 to 3e38 and float16 only
-// from 6e-8 to 65504.  The staged row is therefore scaled by a power of two chosen from
-// its largest magnitude (exact: only the exponent changes), the products are summed in
-// fp32 as usual, and the row sums are scaled back before anything else is added.  The
-// result is what unscaled arithmetic would give wherever that does not overflow, and
-// stays finite and correct where it would.
-
-// Largest biased exponent among eight bfloat16 values.
-__device__ __forceinline__ uint32_t bf16_max_exp8(uint4 v) {
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-    uint32_t e = 0;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        e = max(e, (w[q] >> 7) & 0xffu);
-        e = max(e, (w[q] >> 23) & 0xffu);
-    }
-    return e;
-}
-
-// Maximum over the workgroup; slots = one LDS word per wavefront.  One barrier.
-__device__ __forceinline__ uint32_t workgroup_max(uint32_t v, uint32_t *slots, int tid,
-                                                  int nthreads) {
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) v = max(v, (uint32_t)__shfl_xor((int)v, m));
-    if ((tid & 63) == 0) slots[tid >> 6] = v;
-    __syncthreads();
-    uint32_t r = 0;
-    for (int w = 0; w < (nthreads >> 6); ++w) r = max(r, slots[w]);
-    return r;
-}
-
-// Shift that brings a row whose largest biased exponent is emax to magnitudes in [1, 2):
-// the largest value then has 15 binades of float16 range above it and 14 normal (24 in
-// all) below.  Zero rows and non-finite values keep their values (shift 0).
-__device__ __forceinline__ int bf16_row_shift(uint32_t emax) {
-    return (emax == 0 || emax == 255) ? 0 : (int)emax - 127;
-}
-
-// Eight bfloat16 values -> eight float16 values of x * 2^-shift.
-__device__ __forceinline__ uint4 bf16_to_f16_scaled8(uint4 v, int shift) {
-    uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const float lo = ldexpf(bf2f((uint16_t)(w[q] & 0xffffu)), -shift);
-        const float hi = ldexpf(bf2f((uint16_t)(w[q] >> 16)), -shift);
-        w[q] = (uint32_t)f2h(lo) | ((uint32_t)f2h(hi) << 16);
-    }
-    return make_uint4(w[0], w[1], w[2], w[3]);
-}
-
 // xs holds kc bfloat16 values in natural order, written by every thread of the
 // workgroup; converts them in place to float16 of x * 2^-shift and returns the shift.
 // Barriers inside: before (the writes), between, and none after (the caller's next

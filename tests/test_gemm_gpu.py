@@ -91,7 +91,7 @@ def test_gemm_two_streams_residual_bias_every_workgroup_shape(tuning_env, rows):
                         act_dtype=act_dtype, device=DEV)
         x = make_x(M, K, seed=13, dtype=act_dtype)
         y = _dual(w, x).cpu()
-        ref = _exact(w, x.to(lut_dtype)).to(act_dtype)
+        ref = _exact(w, x).to(act_dtype)
         assert rel_l2(y, ref) <= (TOL if act_dtype == torch.float16 else TOL_BF16)
 
 
@@ -108,7 +108,7 @@ def test_gemm_direct_activations_match_the_pre_pass(tuning_env, M, N, K, gs, act
     x = make_x(M, K, seed=17, dtype=act)
     xd = x.to(DEV)
     y = _dual(w, xd)
-    assert rel_l2(y.cpu(), _exact(w, x.to(lut)).to(act)) <= (TOL if act == torch.float16 else TOL_BF16)
+    assert rel_l2(y.cpu(), _exact(w, x).to(act)) <= (TOL if act == torch.float16 else TOL_BF16)
     tuning_env("FLUTE_GEMM_NO_DIRECT", "1")
     assert torch.equal(_dual(w, xd), y)
     tuning_env("FLUTE_GEMM_NO_DIRECT", None)
@@ -150,9 +150,7 @@ def test_gemm_dtype_mixes(lut_dtype, act_dtype):
     x = make_x(M, K, seed=3, dtype=act_dtype)
     y = _dual(w, x).cpu()
     assert y.dtype == act_dtype
-    # the activations are presented to the matrix cores in the LUT's type
-    xr = x.to(lut_dtype)
-    ref = _exact(w, xr).to(act_dtype)
+    ref = _exact(w, x).to(act_dtype)                   # the reference forward uses x.float()
     tol = TOL if act_dtype == torch.float16 else TOL_BF16
     assert rel_l2(y, ref) <= tol
 
@@ -207,3 +205,35 @@ def test_gemm_full_size_linearity():
     assert rel_l2(y[5:6], y1) <= TOL
     z = run((2.0 * x[:64].float() + x[64:128].float()).half())
     assert rel_l2(z, 2.0 * y[:64].float() + y[64:128].float()) <= 3e-3
+
+
+@pytest.mark.parametrize("kind", ["outliers", "tiny", "huge", "mixed"])
+@pytest.mark.parametrize("M,rows", [(8, None), (40, None), (130, "64"), (300, "128")])
+def test_gemm_bf16_activations_beyond_the_float16_range(tuning_env, kind, M, rows):
+    """bfloat16 rows that float16 cannot hold (|x| > 65504 or < 6e-8) in front of a float16
+    LUT: every row is scaled by its own power of two before it meets the matrix cores and
+    scaled back afterwards, so the result is the reference forward's (x.float() @ W.t()),
+    never inf or 0.  Rows of very different magnitude share a launch."""
+    if rows:
+        tuning_env("FLUTE_GEMM_ROWS", rows)
+    N, K = 256, 1024
+    w = make_weight(N, K, 4, 128, seed=29, act_dtype=torch.bfloat16, device=DEV)
+    x = make_x(M, K, seed=31, dtype=torch.float32)
+    if kind == "outliers":
+        x[::3, 5] = 1.0e5
+        x[1, K - 1] = -3.0e5
+    elif kind == "tiny":
+        x *= 1.0e-7
+    elif kind == "huge":
+        x[: M // 2] *= 1.0e30
+    else:
+        x[::2] *= 1.0e-6
+        x[1::2, ::64] *= 1.0e5
+    x = x.to(torch.bfloat16)
+    y = _dual(w, x).cpu()
+    assert torch.isfinite(y).all()
+    ref = O.linear_reference(x, w["blob"].numpy(), w["lut"], N, K, 128, 4)   # same rounding point
+    assert torch.isfinite(ref).all()
+    # row by row: a launch-wide norm would let the large rows hide the small ones
+    for m in range(M):
+        assert rel_l2(y[m], ref[m]) <= 2e-3, f"row {m}"

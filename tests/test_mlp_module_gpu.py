@@ -264,10 +264,9 @@ def test_gemm_with_rotation_through_the_c_abi(M, lda_pad, act, lut, rank):
                                  torch.cuda.current_stream().cuda_stream)
         assert st == 0, _lib.last_error()
         xr = O.block_fht_reference(x, 128, signs) if block else O.fht_reference(x, signs)
-        # the rotated activations are rounded to the activation type before the GEMM, then
-        # cast to the LUT's type (exact for these magnitudes)
+        # the rotated activations are rounded to the activation type before the GEMM
         xr = xr.to(act)
-        ref = O.linear_exact(xr.to(lut), w["blob"].numpy(), w["lut"], N, K, w["gs"], w["bits"],
+        ref = O.linear_exact(xr, w["blob"].numpy(), w["lut"], N, K, w["gs"], w["bits"],
                              None, None, 0, None, None, None).double()
         if rank:
             ref = ref + (xr.double() @ w["resB"].double().t()) @ w["resA"].double().t()
