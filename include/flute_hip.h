@@ -169,6 +169,21 @@ flute_status flute_gemm(const flute_linear *w, const void *A, void *C, int M,
                         int64_t lda, int64_t ldc, int act_dtype, void *stream);
 
 /*
+ * Scalar differential twin of the LUT GEMM:  C[M, N] = A[M, K] @ W^T for one stream, one
+ * thread per output, every weight decoded from its bit position and looked up in the LUT
+ * in global memory, fp32 sum in ascending k, one rounding.  Shares no code with
+ * flute_gemm.  Replaces qgemm_debug_simple (src/bindings.cpp:243,
+ * src/kernel_debug_simple.cu:94-267).  layout 0: q holds the LOGICAL packed rows
+ * [N, K*bits/8], LSB-first along k (upstream's twin consumes this layout); layout 1: q is
+ * the idxN blob, so the twin and flute_gemm can read the same bytes.  Slow by design.
+ */
+flute_status flute_gemm_debug_simple(const void *q, int64_t q_bytes, int layout,
+                                     const void *lut, int lut_rows, int lut_dtype, int bits,
+                                     int group_size, int N, int K, const void *A, void *C,
+                                     int M, int64_t lda, int64_t ldc, int act_dtype,
+                                     void *stream);
+
+/*
  * Dequantise one stream to a dense row-major [N, K] matrix in lut_dtype,
  * through the same tile decoder the GEMM uses.  which = 1 or 2.  Serves the
  * bit-exact tile check that upstream runs against dequantize_reference

@@ -1,5 +1,7 @@
 """Reader of palettized weight artifacts: one metadata record + the raw member
-files of an artifact directory -> a PalettizedLinear or a SplitQKV.
+files of an artifact directory -> a PalettizedLinear, a SplitQKV or a
+PalettizedEmbedding, and the swap of a built model's layers for them
+(replace_linear_with_palettized, upstream :2921-3026).
 
 Mirrors the upstream reader (src/scripts/palettized_modules.py:229-330 for the
 name/layout rules, :2411-2483 `_read_indices_and_lut`, :2486-2500 `_read_residual`,
@@ -25,9 +27,12 @@ import numpy as np
 import torch
 from torch import nn
 
-from palettized_modules import PalettizedLinear, SplitQKV
+from palettized_modules import (PalettizedEmbedding, PalettizedLinear, SplitQKV,
+                                install_fused_mlp)
 
-__all__ = ["validate_indices_layout", "load_palettized_weight", "LAYOUT_AUDIT", "GS_MISMATCHES"]
+__all__ = ["validate_indices_layout", "load_palettized_weight", "load_palettized_embedding",
+           "load_tied_pair", "load_metadata", "get_layers", "resolve_module",
+           "replace_linear_with_palettized", "LAYOUT_AUDIT", "GS_MISMATCHES"]
 
 LAYOUT_AUDIT = {"idx4": 0, "idxN": 0}     # how many members of each kind were validated
 GS_MISMATCHES = []                         # (ctx, recorded gs, derived gs): stale metadata seen
@@ -250,3 +255,168 @@ def load_palettized_weight(tensor_meta: Dict, artifacts_dir: str, bias=None,
         if off != bias.shape[0]:
             raise ValueError(f"{var}: bias length {bias.shape[0]} != sum of component N ({off})")
     return SplitQKV(*comps)
+
+
+def load_palettized_embedding(tensor_meta: Dict, artifacts_dir: str, residual: bool = True,
+                              verify_sha: bool = True, reference: bool = True):
+    """PalettizedEmbedding for one record (scripts/palettized_modules.py:2731-2767 upstream):
+    both declared streams, every member checked against its sha256, the residual pair when
+    asked for and present, the rotation record of a tied head.  QKV components are refused:
+    an embedding is a single matrix."""
+    var = tensor_meta.get("var", "?")
+    if "components" in tensor_meta:
+        raise ValueError(f"{var}: an embedding record carries no QKV components")
+    indices, lut, bw, gs, N, K = _read_indices_and_lut(tensor_meta, artifacts_dir, var, None,
+                                                       verify_sha)
+    resA = resB = None
+    if residual:
+        resA, resB = _read_residual(tensor_meta, artifacts_dir, var, N, K)
+    indices2 = lut2 = bw2 = None
+    if tensor_meta.get("streams"):
+        indices2, lut2, bw2 = _read_stream2(tensor_meta, artifacts_dir, var, N, K, bw, gs,
+                                            verify_sha)
+    rot = tensor_meta.get("rotation")
+    return PalettizedEmbedding(indices, lut, bw, gs, N, K, indices2=indices2, lut2=lut2,
+                               bitwidth2=bw2, resA=resA, resB=resB,
+                               rotation_seed=rot["seed"] if rot else None,
+                               rotation_k=rot["k"] if rot else None, reference=reference)
+
+
+def _member_rows(meta: Dict):
+    """Every (member, file, digest) a record names: what two consumers of one tied artifact
+    set must agree on."""
+    rows = [("index_file", meta.get("index_file"), meta.get("sha256_idx")),
+            ("lut_file", meta.get("lut_file"), meta.get("sha256_lut"))]
+    for i, entry in enumerate(meta.get("streams") or []):
+        rows += [(f"streams[{i}]", entry.get("file"), entry.get("sha256")),
+                 (f"streams[{i}].lut", entry.get("file"), entry.get("sha256_lut"))]
+    res = meta.get("residual") or {}
+    if res:
+        rows += [("resA", res.get("resA_file"), res.get("sha256_resA")),
+                 ("resB", res.get("resB_file"), res.get("sha256_resB"))]
+    return rows
+
+
+def load_tied_pair(lm_head_meta: Dict, embed_meta: Optional[Dict], artifacts_dir: str,
+                   residual: bool = True, reference: bool = False, verify_sha: bool = True,
+                   awq_scales: Optional[Dict] = None):
+    """(PalettizedLinear, PalettizedEmbedding) over ONE artifact set (upstream :2792-2863):
+    the set is read once through the lm_head record, which must say "tied": true, and the
+    embedding is built on the same tensors; it inherits the head's rotation record, so its
+    gather un-rotates the rows.  When the embedding has a record of its own it must name
+    the same members with the same digests."""
+    var = str(lm_head_meta.get("var", "?"))
+    if lm_head_meta.get("tied") is not True:
+        raise ValueError(f"load_tied_pair({var}): the lm_head record is not marked \"tied\": true")
+    if "components" in lm_head_meta:
+        raise ValueError(f"load_tied_pair({var}): a tied head is a single matrix")
+    if embed_meta is not None and _member_rows(embed_meta) != _member_rows(lm_head_meta):
+        raise ValueError(f"load_tied_pair({var}, {embed_meta.get('var', '?')}): the two records "
+                         f"describe different artifact sets")
+    lm = load_palettized_weight(lm_head_meta, artifacts_dir, residual=residual,
+                                reference=reference, verify_sha=verify_sha, awq_scales=awq_scales)
+    rot = lm_head_meta.get("rotation")
+    emb = PalettizedEmbedding(lm.indices, lm.lut, lm.bitwidth, lm.group_size, lm.N, lm.K,
+                              indices2=lm.indices2, lut2=lm.lut2,
+                              bitwidth2=lm.bitwidth2 if lm.has_stream2 else None,
+                              resA=lm.resA, resB=lm.resB,
+                              rotation_seed=rot["seed"] if rot else None,
+                              rotation_k=rot["k"] if rot else None, reference=reference)
+    return lm, emb
+
+
+_HEADS = ("model.lm_head.weight", "model.embed_tokens.weight")
+
+
+def load_metadata(artifacts_dir: str) -> Dict:
+    """metadata.json of an artifact directory (upstream :3114-3117)."""
+    import json
+    with open(os.path.join(artifacts_dir, "metadata.json")) as f:
+        return json.load(f)
+
+
+def get_layers(model):
+    """The decoder layer list of a causal LM or of a multimodal wrapper (upstream :2866)."""
+    inner = getattr(model, "model", None)
+    if inner is not None and hasattr(inner, "layers"):
+        return inner.layers
+    if inner is not None and hasattr(inner, "language_model"):
+        return inner.language_model.layers
+    raise AttributeError("Cannot find decoder layers in model structure")
+
+
+def resolve_module(model, tensor_name: str):
+    """(holder module, attribute name) of the module a metadata tensor name refers to
+    (upstream :2874-2918): `model.layers.<i>.<path>.weight` inside the layer list,
+    `model.lm_head.weight` / `model.embed_tokens.weight` on the wrapper or on its text model
+    (two different modules of that name are refused)."""
+    parts = tensor_name.split(".")
+    if len(parts) == 3 and parts[0] == "model" and parts[2] == "weight" and \
+            parts[1] in ("lm_head", "embed_tokens"):
+        name = parts[1]
+        holders = [h for h in (model, getattr(model, "model", model)) if hasattr(h, name)]
+        if not holders:
+            raise ValueError(f"resolve_module({tensor_name}): the model has no {name!r}")
+        if any(getattr(h, name) is not getattr(holders[0], name) for h in holders[1:]):
+            raise ValueError(f"resolve_module({tensor_name}): ambiguous, the wrapper and the "
+                             f"text model hold different {name!r} modules")
+        return holders[0], name
+    if len(parts) < 5 or parts[0] != "model" or parts[1] != "layers" or parts[-1] != "weight":
+        raise ValueError(f"resolve_module({tensor_name}): expected model.layers.<i>.<path>.weight")
+    parent = get_layers(model)[int(parts[2])]
+    for attr in parts[3:-2]:
+        parent = getattr(parent, attr)
+    return parent, parts[-2]
+
+
+def replace_linear_with_palettized(model, metadata: Dict, artifacts_dir: str,
+                                   residual: bool = False, reference: bool = False,
+                                   verify_sha: bool = True, awq_scales: Optional[Dict] = None,
+                                   heads_dir: Optional[str] = None):
+    """Swap every module that metadata["tensors"] names for its palettized counterpart
+    (upstream :2921-3026): linear layers (a fused QKV record becomes a SplitQKV), the
+    embedding, a tied head pair from one artifact set; with heads_dir the two head records
+    come from that directory's metadata instead.  A bias of the replaced layer is kept.
+    Afterwards every gated MLP whose gate and up are palettized is wrapped for the merged
+    decode launch (FLUTE_NO_MERGE=1 skips that).  Returns the model."""
+    tensors = dict(metadata["tensors"])
+    if heads_dir is not None:
+        heads = load_metadata(heads_dir)["tensors"]
+        for key in _HEADS:
+            tensors.pop(key, None)
+            if key in heads:
+                tensors[key] = heads[key]
+    compensated = 0
+    for name, meta in tensors.items():
+        src = heads_dir if (heads_dir is not None and name in _HEADS) else artifacts_dir
+        if name == "model.lm_head.weight" and meta.get("tied") is True:
+            lm, emb = load_tied_pair(meta, None, src, residual=residual, reference=reference,
+                                     verify_sha=verify_sha, awq_scales=awq_scales)
+            holder, leaf = resolve_module(model, name)
+            setattr(holder, leaf, lm)
+            holder, leaf = resolve_module(model, "model.embed_tokens.weight")
+            setattr(holder, leaf, emb)
+            compensated += getattr(lm, "fold_order", None) == "rotate_then_awq"
+            continue
+        holder, leaf = resolve_module(model, name)
+        old = getattr(holder, leaf)
+        if name == "model.embed_tokens.weight":
+            new = load_palettized_embedding(meta, src, residual=residual, verify_sha=verify_sha,
+                                            reference=reference)
+        else:
+            bias = getattr(old, "bias", None)
+            new = load_palettized_weight(meta, src, bias=None if bias is None else bias.data,
+                                         residual=residual, reference=reference,
+                                         verify_sha=verify_sha, awq_scales=awq_scales)
+            members = (new.q_proj, new.k_proj, new.v_proj) if isinstance(new, SplitQKV) else (new,)
+            compensated += sum(getattr(m, "fold_order", None) == "rotate_then_awq"
+                               for m in members)
+        setattr(holder, leaf, new)
+    if compensated:
+        print(f"  [ROT] rotate-then-AWQ fold order compensated on {compensated} tensor group(s)",
+              flush=True)
+    fused = install_fused_mlp(model)
+    if fused:
+        print(f"  [merge] FusedPalettizedMLP installed on {fused} MLP group(s) "
+              f"(FLUTE_NO_MERGE=1 disables)", flush=True)
+    return model

@@ -426,12 +426,39 @@ def qgemm_dual_stream(A, indices, lut, bitwidth, indices2, lut2, bitwidth2, resB
                  resB, resA, bias, group_size)
 
 
-def qgemm_debug_simple(A, indices, lut, bitwidth, group_size):
-    """Upstream's scalar-staging differential twin consumes the LOGICAL packed
-    layout (src/kernel_debug_simple.cu).  Its role here is taken by
-    dequant_idxn + a dense matmul in the tests; the entry itself is refused."""
-    _fail("qgemm_debug_simple: the logical-layout twin is not built; use dequant_idxn for "
-          "differential checks")
+def qgemm_debug_simple(A, indices, lut, bitwidth, group_size, q_layout: int = 0):
+    """Scalar differential twin of the GEMM (src/kernel_debug_simple.cu:94-267 upstream):
+    one thread per output, no matrix cores, no LDS.  Like upstream's twin it consumes the
+    LOGICAL packed layout, indices [N, K*bitwidth/8] uint8, LSB-first along K; q_layout=1
+    (an extension) reads the idxN blob instead, so that the twin and the fast kernel can be
+    run on the same bytes."""
+    who = "qgemm_debug_simple"
+    M, K = _check_2d_input(who, A, need_m1=False)
+    b, gs = int(bitwidth), int(group_size)
+    if not 1 <= b <= 4:
+        _fail(f"{who}: bitwidth must be 1, 2, 3 or 4 (got {b})")
+    if indices.dtype != torch.uint8 or not indices.is_contiguous() or not indices.is_cuda:
+        _fail(f"{who}: indices must be a contiguous uint8 tensor on the GPU")
+    if lut.dtype not in _ACT or lut.dim() != 2 or lut.shape[1] != (1 << b) or \
+            not lut.is_contiguous() or lut.device != A.device:
+        _fail(f"{who}: lut must be a contiguous [groups, 2^bitwidth] float16/bfloat16 tensor on "
+              f"the device of A")
+    if K == 0 or (K * b) % 8:
+        _fail(f"{who}: K*bitwidth must be a positive whole number of bytes (K = {K})")
+    row_bytes = K * b // 8
+    N = indices.numel() // row_bytes
+    if N <= 0 or N * row_bytes != indices.numel():
+        _fail(f"{who}: {indices.numel()} index bytes are not N*(K*{b}/8) for any N (K = {K})")
+    if int(q_layout) == 0 and indices.dim() == 2 and tuple(indices.shape) != (N, row_bytes):
+        _fail(f"{who}: logical indices must be [N, K*bitwidth/8] = [{N}, {row_bytes}]")
+    A = A if A.stride(-1) == 1 else A.contiguous()
+    with _on_device_of(A):
+        C = torch.empty((M, N), dtype=A.dtype, device=A.device)
+        check(lib.flute_gemm_debug_simple(indices.data_ptr(), indices.numel(), int(q_layout),
+                                          lut.data_ptr(), lut.shape[0], _ACT[lut.dtype], b, gs, N,
+                                          K, A.data_ptr(), C.data_ptr(), M, A.stride(0) if M else K,
+                                          N, _ACT[A.dtype], _stream_of(A)))
+    return C
 
 
 def qgemm_cutlass_dense(A, W_dense, bitwidth, group_size):

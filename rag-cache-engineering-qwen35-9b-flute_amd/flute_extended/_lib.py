@@ -61,6 +61,8 @@ SYMBOLS = {
     "flute_gemv_multi": (_I, [_LP, _I, _P, ctypes.POINTER(_P), _I, _I, _P]),
     "flute_mlp_block": (_I, [_LP, _LP, _LP, _P, _P, _P, _I, _P]),
     "flute_gemm": (_I, [_LP, _P, _P, _I, ctypes.c_int64, ctypes.c_int64, _I, _P]),
+    "flute_gemm_debug_simple": (_I, [_P, ctypes.c_int64, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _I,
+                                     ctypes.c_int64, ctypes.c_int64, _I, _P]),
     "flute_dequant": (_I, [_LP, _I, _P, _P]),
     "flute_fht": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "flute_embedding": (_I, [_LP, _P, ctypes.c_int64, _P, _P]),

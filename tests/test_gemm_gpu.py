@@ -237,3 +237,46 @@ def test_gemm_bf16_activations_beyond_the_float16_range(tuning_env, kind, M, row
     # row by row: a launch-wide norm would let the large rows hide the small ones
     for m in range(M):
         assert rel_l2(y[m], ref[m]) <= 2e-3, f"row {m}"
+
+
+@pytest.mark.parametrize("bits,gs", [(1, 128), (2, 64), (3, 128), (4, 128), (4, 16), (3, 32)])
+def test_scalar_twin_differential_chain(bits, gs):
+    """Upstream's differential chain (test_flute.py:172-223): the fast kernel on the idxN
+    blob, the scalar twin on the LOGICAL packed rows and the twin on the blob.  The twin
+    shares no code with the fast path (one thread per output, bit-position decode, LUT in
+    global memory), so agreement means both read the format the same way: the two twin
+    layouts must agree bit for bit (same sums in the same order), twin and fast kernel
+    within fp32 reassociation, and all three exactly on one-hot rows."""
+    M, K, N = 64, 512, 256
+    w = make_weight(N, K, bits, gs, seed=43 + bits, device=DEV)
+    logical = torch.from_numpy(O.logical_packed_rows(w["idx"].numpy(), bits)).to(DEV)
+    assert logical.shape == (N, K * bits // 8)
+    x = make_x(M, K, seed=44).to(DEV)
+    fast = fx.qgemm_per_group_lut(x, w["blob_d"], w["lut_d"], bitwidth=bits, group_size=gs,
+                                  indices_layout=f"idx{bits}")
+    twin = fx.qgemm_per_group_lut(x, logical, w["lut_d"], bitwidth=bits, group_size=gs,
+                                  backend="debug_simple", indices_layout=f"idx{bits}")
+    twin_blob = fx.qgemm_debug_simple(x, w["blob_d"], w["lut_d"], bits, gs, q_layout=1)
+    assert torch.equal(twin, twin_blob)
+    assert rel_l2(fast.cpu(), twin.cpu()) <= 5e-4
+    assert rel_l2(twin.cpu(), _exact(w, x.cpu()).half()) <= TOL
+    eye = torch.eye(K, dtype=torch.float16, device=DEV)
+    W = O.dequant(w["blob"].numpy(), w["lut"], N, K, gs, bits).t().half()
+    assert torch.equal(fx.qgemm_debug_simple(eye, logical, w["lut_d"], bits, gs).cpu(), W)
+    assert torch.equal(fx.qgemm_debug_simple(eye, w["blob_d"], w["lut_d"], bits, gs, q_layout=1).cpu(), W)
+    assert torch.equal(fx.qgemm_per_group_lut(eye, w["blob_d"], w["lut_d"], bitwidth=bits,
+                                              group_size=gs, indices_layout=f"idx{bits}").cpu(), W)
+
+
+def test_scalar_twin_refusals_and_bf16():
+    w = make_weight(256, 128, 4, 128, seed=47, lut_dtype=torch.bfloat16, device=DEV)
+    x = make_x(3, 128, seed=48, dtype=torch.bfloat16).to(DEV)
+    y = fx.qgemm_debug_simple(x, w["blob_d"], w["lut_d"], 4, 128, q_layout=1)
+    assert y.dtype == torch.bfloat16
+    assert rel_l2(y.cpu(), _exact(w, x.cpu()).bfloat16()) <= TOL
+    with pytest.raises(RuntimeError):
+        fx.qgemm_debug_simple(x, w["blob_d"][:-1], w["lut_d"], 4, 128)        # truncated
+    with pytest.raises(RuntimeError):
+        fx.qgemm_debug_simple(x, w["blob_d"], w["lut_d"][:, :8], 4, 128)      # wrong LUT width
+    with pytest.raises(RuntimeError):
+        fx.qgemm_debug_simple(x, w["blob_d"], w["lut_d"], 5, 128)
