@@ -1,20 +1,23 @@
 #!/usr/bin/env python3
-"""Benchmark of the idxN LUT-palettized decode path on one MI355X.
+"""Benchmark of the idxN LUT-palettized linear layer on one MI355X.
 
-One step = one token through the fused MLP block of the benchmark's second
-configuration: gate and up projections 4096 -> 12288 (one merged launch with
-the SiLU*mul epilogue), then the down projection 12288 -> 4096; idx4 blobs,
-group 128, fp16 LUTs, bf16 activations, M = 1.  The weights of a step live in
-HBM before the clock starts; consecutive steps use different weight sets whose
-total size exceeds three times the 256 MB Infinity Cache, so every step streams
-its 72 MiB from HBM.
+Headline (`value`, `ms_per_step`, `roofline`): the M = 1 LUT GEMV of the MLP up-projection,
+K = 4096 -> N = 12288, idx4 blob, group 128, fp16 LUT, bf16 activations.  One step = one
+call of flute_gemv.  The weights live in HBM before the clock starts and consecutive steps
+use different weights whose total size exceeds three times the 256 MB memory-side cache,
+so every step streams its 24 MiB from HBM ("cold").  `value` = packed index + LUT bytes
+per second (the numerator the target is stated on); `roofline.achieved` counts all
+algorithmic bytes of the launch (indices, LUT, activations in, outputs).
 
-Prints ONE JSON line.  `value` is algorithmic bytes (packed indices + LUTs +
-activations in and out) per second over exactly `--steps` steps, timed with
-events on the stream the kernels run on.  `roofline` describes the dominant
-kernel (the merged gate+up GEMV) from a second timed region that launches only
-that kernel; `cpu_baseline` times the oracle's restatement of the upstream
-torch path on the host for a bounded sample.
+Timing: the K steps are captured into one hipGraph; the graph is replayed 21 times with
+events on the launch stream and the median replay is reported (time of exactly K steps).
+
+Beside it, in the same JSON line: `mlp_block` (the fused MLP decode block of the second
+configuration: merged gate+up with SiLU*mul, then down), `gemm` (the M > 1 LUT-GEMM, both
+shapes, M = 16 / 64 / 256 / 1024), `other_m1_configs` (cache-resident, fused rotation,
+lm_head, narrow shapes with the K splits swept) and `cpu_baseline` (the oracle's
+restatement of the upstream torch path on the host cores, bounded samples).
+Every row is parity-gated against the oracle; a row whose gate fails aborts the run.
 """
 from __future__ import annotations
 
@@ -30,10 +33,22 @@ sys.path[:0] = [os.path.join(ROOT, "rag-cache-engineering-qwen35-9b-flute_amd")]
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0      # MI355X published dense bf16/fp16 MFMA rate
 H, I, GS = 4096, 12288, 128
-# HBM bytes one launch of the merged gate+up kernel moves, from FETCH_SIZE and WRITE_SIZE
-# counter runs of this file scaled by a copy of known size (--calibrate-copy); the readings
-# are kept in profiles/gemv4_gate_up_hbm_traffic.txt.  Only valid for the default workload.
-TRAFFIC_GATE_UP_BYTES = 50790600
+# HBM bytes one launch of the headline kernel moves come from FETCH_SIZE and WRITE_SIZE counter
+# runs of this file under rocprofv3 (scaled by a copy of known size, --calibrate-copy); a
+# counter cannot be read from inside the process, so the figure is read back from the summary
+# those runs left in profiles/ (a line "traffic_bytes_per_launch: N"), null when it is absent.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemv4_4096x12288_hbm_traffic.txt")
+REPLAYS = 21
+
+
+def _traffic_from_profile():
+    try:
+        for line in open(TRAFFIC_FILE):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def _weights(torch, N, K, gen, dev, lut_dtype):
@@ -52,9 +67,9 @@ def _desc(_lib, blob, lut, N, K):
     return d
 
 
-def _time_graph(torch, fn, reps=3):
-    """Capture fn() (a sequence of launches on the current stream) once, replay it
-    `reps` times, return the best elapsed milliseconds of one replay."""
+def _time_graph(torch, fn, reps=REPLAYS):
+    """Capture fn() (a sequence of launches on the current stream) once, replay it `reps`
+    times, return the median elapsed milliseconds of one replay."""
     fn()
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
@@ -62,7 +77,7 @@ def _time_graph(torch, fn, reps=3):
         fn()
     graph.replay()
     torch.cuda.synchronize()
-    best = float("inf")
+    times = []
     for _ in range(reps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
@@ -70,95 +85,129 @@ def _time_graph(torch, fn, reps=3):
         graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        best = min(best, e0.elapsed_time(e1))
-    return best
+        times.append(e0.elapsed_time(e1))
+    times.sort()
+    return times[len(times) // 2]
 
 
-def _cpu_baseline(torch, seconds_budget=12.0):
-    """The upstream reference path as shipped (unpack the blob, gather the LUT,
-    fp32 matmul; scripts/palettized_modules.py:811-824, 1241-1251 upstream) through
-    the oracle, on the benchmark's first configuration: M=1, 4096 -> 4096, fp16."""
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _cpu_baseline(torch):
+    """The upstream reference path through the oracle, on the host cores, bounded samples:
+    (i) as shipped: unpack the blob, gather the LUT, fp32 matmul on every call
+        (scripts/palettized_modules.py:811-824, 1241-1251 upstream);
+    (ii) cached logical indices: gather + matmul (:668-705);
+    (iii) cached fp32 weight: the matmul alone, the best case.
+    The headline workload (M = 1, 4096 -> 12288) gives `value`; the first configuration
+    (4096 -> 4096, fp16) is listed with all three variants."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import flute_oracle as O
-    from flute_extended import idxN
-    N = K = 4096
-    g = torch.Generator().manual_seed(0)
-    idx = torch.randint(0, 16, (N, K), generator=g, dtype=torch.uint8)
-    blob = idxN.pack_idxn(idx.numpy(), 4)
-    lut = (torch.randn(N // GS, 16, generator=g) * 0.02).sort(dim=1).values.half()
-    x = torch.randn(1, K, generator=g).half()
-    O.linear_reference(x, blob, lut, N, K, GS, 4)
-    times = []
-    t_end = time.perf_counter() + seconds_budget
-    # a bounded sample: about twelve seconds of host work (at least three calls)
-    while time.perf_counter() < t_end or len(times) < 3:
-        t0 = time.perf_counter()
-        O.linear_reference(x, blob, lut, N, K, GS, 4)
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
-    nbytes = N * K // 2 + lut.numel() * 2 + K * 2 + N * 2
-    return {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"M=1 4096->4096 idx4 gs128 fp16, as shipped (unpack+gather+fp32 matmul per "
-                      f"call), median of {len(times)} calls, {med * 1e3:.1f} ms/call, "
-                      f"os.cpu_count={os.cpu_count()}"}
+    import numpy as np
+
+    def sample(fn, budget, at_least=3, at_most=40):
+        fn()
+        times, t_end = [], time.perf_counter() + budget
+        while (time.perf_counter() < t_end or len(times) < at_least) and len(times) < at_most:
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    def variants(N, K, dtype, budget):
+        g = torch.Generator().manual_seed(N + K)
+        blob = torch.randint(0, 256, (N * K // 2,), dtype=torch.uint8, generator=g).numpy()
+        lut = (torch.randn(N // GS, 16, generator=g) * 0.02).sort(dim=1).values.half()
+        x = torch.randn(1, K, generator=g).to(dtype)
+        nbytes = N * K // 2 + lut.numel() * 2
+        idx = torch.from_numpy(O.unpack_idxn(blob, N, K, 4).astype(np.int64))
+        rows = torch.arange(N) // GS
+        W = lut[rows].float().gather(1, idx)
+        out = {}
+        for name, fn in (
+                ("as_shipped", lambda: O.linear_reference(x, blob, lut, N, K, GS, 4)),
+                ("cached_indices", lambda: (x.float() @ lut[rows].float().gather(1, idx).t()).to(dtype)),
+                ("cached_fp32_weight", lambda: (x.float() @ W.t()).to(dtype))):
+            med, n = sample(fn, budget)
+            out[name] = {"ms_per_call": round(med * 1e3, 3), "gbs_index_plus_lut": round(nbytes / med / 1e9, 4),
+                         "calls": n}
+        return out
+
+    head = variants(I, H, torch.bfloat16, 4.0)
+    first = variants(H, H, torch.float16, 2.0)
+    return {"value": head["as_shipped"]["gbs_index_plus_lut"], "unit": "GB/s",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"M=1 4096->12288 idx4 gs128, fp16 LUT, bf16 activations, upstream reference path as "
+                      f"shipped (unpack + gather + fp32 matmul per call), median of "
+                      f"{head['as_shipped']['calls']} calls, {head['as_shipped']['ms_per_call']} ms/call",
+            "cpu_model": _cpu_model(), "os_cpu_count": os.cpu_count(),
+            "torch_threads": torch.get_num_threads(),
+            "variants_4096x12288_bf16": head, "variants_config0_4096x4096_fp16": first}
 
 
-def _gemv_section(torch, _lib, ctypes, sets, gen, dev, O):
-    """The other M = 1 configurations beside the headline block, each parity-gated against
-    the oracle on the rows of one tile: the north-star GEMV 4096 -> 12288 (GB/s on packed
-    index + LUT bytes, the numerator the target is stated on), the same GEMV with the
-    block-128 Hadamard rotation fused into its prologue, and the narrow shapes of the split-K
-    configuration."""
-    out = {}
-    act = torch.bfloat16
-    x = torch.randn(1, H, device=dev, generator=gen).to(act)
-    stream = lambda: torch.cuda.current_stream().cuda_stream
+def _oracle_rows(O, blob, lut, K, tile):
+    """The 128 rows of one tile, dequantised by the oracle from the blob bytes (fp64)."""
+    per = (K // 64) * 4096
+    sub = blob[tile * per:(tile + 1) * per].cpu().numpy()
+    return O.dequant(sub, lut[tile:tile + 1].cpu(), 128, K, GS, 4).double()
 
-    def run(name, descs, N, K, xin, keep, signs=None, block=0, split=0):
-        y = torch.zeros(1, N, dtype=act, device=dev)
+
+def _rel(got, ref):
+    return float(((got - ref) ** 2).sum() / (ref ** 2).sum()) ** 0.5
+
+
+class _Gemv:
+    """flute_gemv over a rotation of weights of one shape, parity-gated against the oracle."""
+
+    def __init__(self, torch, _lib, ctypes, O, dev, act):
+        self.torch, self.lib, self.ct, self.O, self.dev, self.act = torch, _lib, ctypes, O, dev, act
+
+    def run(self, name, descs, keep, N, K, x, signs=None, block=0, split=0, launches=None):
+        torch, _lib, ctypes = self.torch, self.lib, self.ct
+        y = torch.zeros(1, N, dtype=self.act, device=self.dev)
 
         def call(i):
-            st = _lib.lib.flute_gemv(ctypes.byref(descs[i % len(descs)]), xin.data_ptr(),
-                                     y.data_ptr(), _lib.BF16, split, stream())
+            st = _lib.lib.flute_gemv(ctypes.byref(descs[i % len(descs)]), x.data_ptr(), y.data_ptr(),
+                                     _lib.BF16, split, torch.cuda.current_stream().cuda_stream)
             if st != 0:
                 raise RuntimeError(_lib.last_error())
 
         call(0)
         torch.cuda.synchronize()
         blob, lut = keep[0]
-        per = (K // 64) * 4096
-        tile = (N // 128) // 2
-        Wt = O.dequant(blob[tile * per:(tile + 1) * per].cpu().numpy(), lut[tile:tile + 1].cpu(),
-                       128, K, GS, 4).double()
-        xr = xin.cpu()
+        xr = x.cpu()
         if signs is not None:
-            xr = O.block_fht_reference(xr, block, signs.cpu()).to(act)
-        ref = xr.double() @ Wt.t()
-        got = y[:, tile * 128:(tile + 1) * 128].cpu().double()
-        err = float(((got - ref) ** 2).sum() / (ref ** 2).sum()) ** 0.5
+            xr = self.O.block_fht_reference(xr, block, signs.cpu()).to(self.act)
+        tiles = sorted({0, (N // 128) // 2, N // 128 - 1})
+        ref = torch.cat([xr.double() @ _oracle_rows(self.O, blob, lut, K, t).t() for t in tiles], 1)
+        got = torch.cat([y[:, t * 128:(t + 1) * 128] for t in tiles], 1).cpu().double()
+        err = _rel(got, ref)
+        floor = _rel(ref.to(self.act).double(), ref)           # what one bf16 rounding costs by itself
         if err > 4e-3:
             raise SystemExit(f"bench.py: parity gate failed for {name} ({err:.2e})")
-        n = max(96, len(descs))                     # every weight of the rotation once per replay
-        us = _time_graph(torch, lambda: [call(i) for i in range(n)]) / n * 1e3
+        n = launches or max(96, len(descs))
+        ms = _time_graph(torch, lambda: [call(i) for i in range(n)])
+        us = ms / n * 1e3
         wbytes = N * K // 2 + (N // GS) * 32
-        out[name] = {"us_per_call": round(us, 2), "gbs_index_plus_lut": round(wbytes / us / 1e3, 1),
-                     "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                     "parity_rel_l2": err}
+        return {"us_per_call": round(us, 3), "gbs_index_plus_lut": round(wbytes / us / 1e3, 1),
+                "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), "parity_rel_l2": err,
+                "output_rounding_alone": floor, "launches_per_replay": n}
 
-    # 4096 -> 12288 weights: the gate and up projections of the sets plus as many more as it
-    # takes to rotate through more than three times the 256 MB memory-side cache
-    gate = [s["g"] for s in sets] + [s["u"] for s in sets]
-    keep = [s["t"][0] for s in sets] + [s["t"][1] for s in sets]
-    while len(gate) * (I * H // 2) < 3.1 * 256 * 2 ** 20:
-        b, l = _weights(torch, I, H, gen, dev, torch.float16)
-        keep.append((b, l))
-        gate.append(_desc(_lib, b, l, I, H))
-    run("gemv_4096x12288", gate, I, H, x, keep)
-    out["gemv_4096x12288"]["weights_in_rotation"] = len(gate)
-    # the same launch on one weight only: 25 MB stay resident in the memory-side cache
-    run("gemv_4096x12288_cache_resident", gate[:1], I, H, x, keep[:1])
+
+def _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, x):
+    """The other M = 1 rows: the same launch on one weight only (cache-resident), the
+    block-128 Hadamard rotation fused into the prologue, the lm_head shape, and the narrow
+    shapes of the split-K configuration (the library's own choice and K splits 2/4/8)."""
+    out = {}
+    out["gemv_4096x12288_cache_resident"] = gv.run("cache_resident", gate[:1], keep[:1], I, H, x)
     signs = (torch.randint(0, 2, (H,), device=dev, generator=gen).float() * 2 - 1).contiguous()
     rot = []
     for g in gate:
@@ -166,133 +215,174 @@ def _gemv_section(torch, _lib, ctypes, sets, gen, dev, O):
         ctypes.memmove(ctypes.byref(d), ctypes.byref(g), ctypes.sizeof(d))
         d.signs, d.rot_block = signs.data_ptr(), 128
         rot.append(d)
-    run("gemv_4096x12288_fht128_fused", rot, I, H, x, keep, signs=signs, block=128)
-    # the widest weight of the model family: lm_head 4096 -> 248320 (0.5 GB of indices, upstream
-    # quotes its plain streamer on this shape); two weights in rotation are 1 GB
-    NV = 248320
+    out["gemv_4096x12288_fht128_fused"] = gv.run("fht128", rot, keep, I, H, x, signs=signs, block=128)
+    NV = 248320                                    # lm_head: 0.5 GB of indices, two in rotation
     ws = [_weights(torch, NV, H, gen, dev, torch.float16) for _ in range(2)]
-    run("gemv_lm_head_4096x248320", [_desc(_lib, b, l, NV, H) for b, l in ws], NV, H, x, ws)
+    out["gemv_lm_head_4096x248320"] = gv.run("lm_head", [_desc(_lib, b, l, NV, H) for b, l in ws], ws,
+                                             NV, H, x, launches=12)
     del ws
-    # narrow outputs: the library's own choice (it does not split K on this device) and the
-    # forced K splits of the configuration beside it; enough weights to stay out of the caches
     for N in (1024, 512):
         count = int(3.1 * 256 * 2 ** 20 // (N * H // 2)) + 1
         ws = [_weights(torch, N, H, gen, dev, torch.float16) for _ in range(count)]
         ds = [_desc(_lib, b, l, N, H) for b, l in ws]
-        name = f"gemv_narrow_4096x{N}"
-        run(name, ds, N, H, x, ws)
-        res = out[name]
+        res = gv.run(f"narrow{N}", ds, ws, N, H, x)
         res["split_chosen"] = int(_lib.lib.flute_pick_split(N, H))
         res["weights_in_rotation"] = count
-        sweep = {}
-        for sp in (2, 4, 8):
-            run("_sweep", ds, N, H, x, ws, split=sp)
-            sweep[str(sp)] = out.pop("_sweep")["us_per_call"]
-        res["us_per_call_forced_split"] = sweep
+        res["us_per_call_forced_split"] = {
+            str(sp): gv.run(f"narrow{N}/split{sp}", ds, ws, N, H, x, split=sp)["us_per_call"]
+            for sp in (1, 2, 4, 8)}
+        out[f"gemv_narrow_4096x{N}"] = res
         del ws, ds
     return out
 
 
-def _gemm_section(torch, _lib, ctypes, sets, gen, dev, O):
-    """The second half of the metric: C[M, 12288] = A[M, 4096] @ W^T on the same idx4
-    blobs (the gate projections of the weight sets), bf16 LUT, bf16 activations, bf16
-    MFMA with fp32 accumulate.  One call = flute_gemm as a caller sees it, including its
-    activation pre-pass.  Headline M = 256; the other M of the configuration are listed."""
-    lut_bf = [(torch.randn(I // GS, 16, device=dev, generator=gen) * 0.02).sort(dim=1).values
-              .to(torch.bfloat16).contiguous() for _ in sets]
-    descs = []
-    for s, lut in zip(sets, lut_bf):
-        blob = s["t"][0][0]
-        descs.append(_desc(_lib, blob, lut, I, H))
-    res = {}
-    for M in (256, 16, 64, 1024):
-        A = torch.randn(M, H, device=dev, generator=gen).to(torch.bfloat16)
-        C = torch.empty(M, I, dtype=torch.bfloat16, device=dev)
+def _mlp_block(torch, _lib, ctypes, O, dev, gen, sets, x, act, steps):
+    """Second configuration: one token through gate+up (one merged launch with SiLU*mul)
+    and down; bytes = indices + LUTs + x, h written and read, y."""
+    h = torch.zeros(1, I, dtype=act, device=dev)
+    y = torch.zeros(1, H, dtype=act, device=dev)
 
-        def call(i):
-            st = _lib.lib.flute_gemm(ctypes.byref(descs[i % len(descs)]), A.data_ptr(), C.data_ptr(),
-                                     M, H, I, _lib.BF16, torch.cuda.current_stream().cuda_stream)
-            if st != 0:
-                raise RuntimeError(_lib.last_error())
+    def block(s):
+        st = _lib.lib.flute_mlp_block(ctypes.byref(s["g"]), ctypes.byref(s["u"]), ctypes.byref(s["d"]),
+                                      x.data_ptr(), h.data_ptr(), y.data_ptr(), _lib.BF16,
+                                      torch.cuda.current_stream().cuda_stream)
+        if st != 0:
+            raise RuntimeError(_lib.last_error())
 
-        call(0)
-        torch.cuda.synchronize()
-        # parity against the oracle's dequantised rows of three tiles, fp64 matmul
-        blob, lut = sets[0]["t"][0][0], lut_bf[0]
-        per = (H // 64) * 4096
-        num = den = 0.0
-        Ad = A.cpu().double()
-        for tile in (0, 41, 95):
-            Wt = O.dequant(blob[tile * per:(tile + 1) * per].cpu().numpy(), lut[tile:tile + 1].cpu(),
-                           128, H, GS, 4).double()
-            ref = Ad @ Wt.t()
-            got = C[:, tile * 128:(tile + 1) * 128].cpu().double()
-            num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
-        err = (num / den) ** 0.5
-        if err > 4e-3:                      # bf16 output: rounding alone is 2^-9
-            raise SystemExit(f"bench.py: GEMM parity gate failed at M={M} ({err:.2e})")
-        n = 48
-        us = _time_graph(torch, lambda: [call(i) for i in range(n)]) / n * 1e3
-        tf = 2.0 * M * I * H / us / 1e6
-        res[M] = {"us_per_call": round(us, 2), "tflops": round(tf, 1),
-                  "frac_mfma": round(tf / MFMA_PEAK_TFLOPS, 4), "parity_rel_l2": err}
+    def gate_up(s):
+        st = _lib.lib.flute_gemv_mlp(ctypes.byref(s["g"]), ctypes.byref(s["u"]), x.data_ptr(),
+                                     h.data_ptr(), _lib.BF16, 0, torch.cuda.current_stream().cuda_stream)
+        if st != 0:
+            raise RuntimeError(_lib.last_error())
+
+    block(sets[0])
+    torch.cuda.synchronize()
+    (gb, gl), (ub, ul), (db, dl) = sets[0]["t"]
+    xd, hd = x.cpu().double(), h.cpu().double()
+    ref_h = torch.cat([O.silu_mul_exact(xd @ _oracle_rows(O, gb, gl, H, t).t(),
+                                        xd @ _oracle_rows(O, ub, ul, H, t).t()) for t in (0, 37, 95)], 1)
+    got_h = torch.cat([hd[:, t * 128:(t + 1) * 128] for t in (0, 37, 95)], 1)
+    ref_y = torch.cat([hd @ _oracle_rows(O, db, dl, I, t).t() for t in (0, 13, 31)], 1)
+    got_y = torch.cat([y.cpu().double()[:, t * 128:(t + 1) * 128] for t in (0, 13, 31)], 1)
+    err_h, err_y = _rel(got_h, ref_h), _rel(got_y, ref_y)
+    if err_h > 4e-3 or err_y > 4e-3:
+        raise SystemExit(f"bench.py: MLP block parity gate failed (h {err_h:.2e}, y {err_y:.2e})")
+    n = len(sets)
+    ms_step = _time_graph(torch, lambda: [block(sets[i % n]) for i in range(steps)]) / steps
+    ms_gu = _time_graph(torch, lambda: [gate_up(sets[i % n]) for i in range(steps)]) / steps
+    lut_bytes = (I // GS) * 32
+    bytes_gate_up = 2 * (I * H // 2 + lut_bytes) + H * 2 + I * 2
+    bytes_down = H * I // 2 + (H // GS) * 32 + I * 2 + H * 2
+    gbs = (bytes_gate_up + bytes_down) / (ms_step * 1e-3) / 1e9
+    return {"workload": "fused MLP decode M=1: gate+up 4096->12288 (merged, SiLU*mul) + down "
+                        "12288->4096, idx4, group 128, fp16 LUT, bf16 activations, cold weights",
+            "us_per_block": round(ms_step * 1e3, 3), "gbs": round(gbs, 1),
+            "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "bytes_per_block": bytes_gate_up + bytes_down,
+            "gate_up_kernel": {"us_per_launch": round(ms_gu * 1e3, 3), "bytes": bytes_gate_up,
+                               "gbs": round(bytes_gate_up / ms_gu / 1e6, 1),
+                               "frac_hbm_peak": round(bytes_gate_up / ms_gu / 1e6 / HBM_PEAK_GBS, 4)},
+            "parity_rel_l2": {"h": err_h, "y": err_y,
+                              "output_rounding_alone": {"h": _rel(ref_h.to(act).double(), ref_h),
+                                                        "y": _rel(ref_y.to(act).double(), ref_y)}},
+            "weight_sets": n}
+
+
+def _gemm_section(torch, _lib, ctypes, O, dev, gen, sets):
+    """The second half of the metric: C[M, N] = A[M, K] @ W^T on idx4 blobs with a bf16 LUT,
+    bf16 activations, bf16 MFMA with fp32 accumulate, for both shapes of the configuration
+    (4096 -> 12288 and 12288 -> 4096) at M = 16 / 64 / 256 / 1024.  One call = flute_gemm as
+    a caller sees it, its activation pre-pass included.  M >= 256 is priced against the
+    matrix-core peak, M = 16 and 64 against HBM (index + LUT + A + C bytes): that is the
+    roof that binds there."""
+    shapes = {}
+    for N, K, which in ((I, H, 0), (H, I, 2)):
+        blobs = [s["t"][which][0] for s in sets]
+        luts = [(torch.randn(N // GS, 16, device=dev, generator=gen) * 0.02).sort(dim=1).values
+                .to(torch.bfloat16).contiguous() for _ in sets]
+        descs = [_desc(_lib, b, l, N, K) for b, l in zip(blobs, luts)]
+        rows = {}
+        for M in (256, 16, 64, 1024):
+            A = torch.randn(M, K, device=dev, generator=gen).to(torch.bfloat16)
+            C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+            def call(i):
+                st = _lib.lib.flute_gemm(ctypes.byref(descs[i % len(descs)]), A.data_ptr(), C.data_ptr(),
+                                         M, K, N, _lib.BF16, torch.cuda.current_stream().cuda_stream)
+                if st != 0:
+                    raise RuntimeError(_lib.last_error())
+
+            call(0)
+            torch.cuda.synchronize()
+            tiles = (0, (N // 128) // 2 - 1, N // 128 - 1)
+            Ad = A.cpu().double()
+            ref = torch.cat([Ad @ _oracle_rows(O, blobs[0], luts[0], K, t).t() for t in tiles], 1)
+            got = torch.cat([C[:, t * 128:(t + 1) * 128] for t in tiles], 1).cpu().double()
+            err = _rel(got, ref)
+            if err > 4e-3:                      # bf16 output: rounding alone is 2^-9
+                raise SystemExit(f"bench.py: GEMM parity gate failed at {K}->{N}, M={M} ({err:.2e})")
+            n = 48
+            us = _time_graph(torch, lambda: [call(i) for i in range(n)]) / n * 1e3
+            tf = 2.0 * M * N * K / us / 1e6
+            nbytes = N * K // 2 + (N // GS) * 32 + 2 * M * (K + N)
+            rows[M] = {"us_per_call": round(us, 2), "tflops": round(tf, 1),
+                       "frac_mfma": round(tf / MFMA_PEAK_TFLOPS, 4),
+                       "gbs": round(nbytes / us / 1e3, 1), "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                       "bound": "mfma" if M >= 256 else "hbm", "parity_rel_l2": err}
+        shapes[f"{K}x{N}"] = rows
     # the rotated-input configuration at M = 8: block-128 Hadamard rotation of the rows in
-    # front of the same GEMM (one rotation launch that writes the operand order + the kernel)
-    M = 8
+    # front of the 4096 -> 12288 GEMM, fp16 LUT, bf16 activations
+    M, N, K = 8, I, H
+    blob = sets[0]["t"][0][0]
+    lut = sets[0]["t"][0][1]
     signs = (torch.randint(0, 2, (H,), device=dev, generator=gen).float() * 2 - 1).contiguous()
     rot = []
-    for d in descs:
+    for s_ in sets:
         r = _lib.FluteLinear()
-        ctypes.memmove(ctypes.byref(r), ctypes.byref(d), ctypes.sizeof(r))
+        ctypes.memmove(ctypes.byref(r), ctypes.byref(s_["g"]), ctypes.sizeof(r))
         r.signs, r.rot_block = signs.data_ptr(), 128
         rot.append(r)
-    A = torch.randn(M, H, device=dev, generator=gen).to(torch.bfloat16)
-    C = torch.empty(M, I, dtype=torch.bfloat16, device=dev)
+    A = torch.randn(M, K, device=dev, generator=gen).to(torch.bfloat16)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
 
     def call_rot(i):
-        st = _lib.lib.flute_gemm(ctypes.byref(rot[i % len(rot)]), A.data_ptr(), C.data_ptr(),
-                                 M, H, I, _lib.BF16, torch.cuda.current_stream().cuda_stream)
+        st = _lib.lib.flute_gemm(ctypes.byref(rot[i % len(rot)]), A.data_ptr(), C.data_ptr(), M, K, N,
+                                 _lib.BF16, torch.cuda.current_stream().cuda_stream)
         if st != 0:
             raise RuntimeError(_lib.last_error())
 
     call_rot(0)
     torch.cuda.synchronize()
-    blob, lut = sets[0]["t"][0][0], lut_bf[0]
-    per = (H // 64) * 4096
     Ar = O.block_fht_reference(A.cpu(), 128, signs.cpu()).to(torch.bfloat16).double()
-    num = den = 0.0
-    for tile in (0, 41, 95):
-        Wt = O.dequant(blob[tile * per:(tile + 1) * per].cpu().numpy(), lut[tile:tile + 1].cpu(),
-                       128, H, GS, 4).double()
-        ref = Ar @ Wt.t()
-        got = C[:, tile * 128:(tile + 1) * 128].cpu().double()
-        num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
-    err = (num / den) ** 0.5
+    tiles = (0, 41, 95)
+    ref = torch.cat([Ar @ _oracle_rows(O, blob, lut, K, t).t() for t in tiles], 1)
+    got = torch.cat([C[:, t * 128:(t + 1) * 128] for t in tiles], 1).cpu().double()
+    err = _rel(got, ref)
     if err > 4e-3:
         raise SystemExit(f"bench.py: rotated GEMM parity gate failed ({err:.2e})")
-    n = 48
-    us = _time_graph(torch, lambda: [call_rot(i) for i in range(n)]) / n * 1e3
-    rotated = {"us_per_call": round(us, 2), "parity_rel_l2": err,
-               "workload": "M=8, block-128 Hadamard rotation of the input + LUT-GEMM 4096->12288"}
-    head = res[256]
-    return {"rotated_input_M8": rotated,
-            "workload": "LUT-GEMM M=256: 4096->12288, idx4, group 128, bf16 LUT, bf16 activations, "
-                        "bf16 MFMA fp32 accumulate; whole flute_gemm call (activation pre-pass + kernel)",
-            "value": head["tflops"], "unit": "TFLOP/s", "peak": MFMA_PEAK_TFLOPS,
-            "frac": head["frac_mfma"], "us_per_call": head["us_per_call"],
-            "parity_rel_l2": head["parity_rel_l2"],
-            "other_M": {str(m): res[m] for m in (16, 64, 1024)}}
+    us = _time_graph(torch, lambda: [call_rot(i) for i in range(48)]) / 48 * 1e3
+    head = shapes[f"{H}x{I}"][256]
+    return {"workload": "LUT-GEMM M=256: 4096->12288, idx4, group 128, bf16 LUT, bf16 activations, bf16 "
+                        "MFMA fp32 accumulate; whole flute_gemm call (activation pre-pass + kernel)",
+            "value": head["tflops"], "unit": "TFLOP/s", "peak": MFMA_PEAK_TFLOPS, "frac": head["frac_mfma"],
+            "us_per_call": head["us_per_call"], "parity_rel_l2": head["parity_rel_l2"],
+            "shapes": {k: {str(m): v[m] for m in (16, 64, 256, 1024)} for k, v in shapes.items()},
+            "rotated_input_M8": {"us_per_call": round(us, 2), "parity_rel_l2": err,
+                                 "workload": "M=8, block-128 Hadamard rotation of the input + LUT-GEMM "
+                                             "4096->12288, fp16 LUT, bf16 activations"}}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=240)
-    ap.add_argument("--warmup", type=int, default=24)
-    ap.add_argument("--sets", type=int, default=12, help="distinct weight sets (72 MiB each)")
+    ap.add_argument("--steps", type=int, default=340)
+    ap.add_argument("--warmup", type=int, default=34)
+    ap.add_argument("--weights", type=int, default=34,
+                    help="distinct 4096->12288 weights in rotation (24 MiB each; 34 = 850 MB)")
+    ap.add_argument("--sets", type=int, default=12, help="MLP weight sets (72 MiB each)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M>1 LUT-GEMM section")
-    ap.add_argument("--no-extra", action="store_true", help="skip the other M=1 configurations")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the MLP block and the other M=1 configurations")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 64 MiB device copy, so that a counter run of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE/WRITE_SIZE by")
@@ -308,11 +398,15 @@ def main():
         return 2
     from flute_extended import _lib          # fails loudly if libflute_hip.so is missing
     import ctypes
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import flute_oracle as O                 # the checker of the parity gates only
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(1234)
     act = torch.bfloat16
 
+    # MLP weight sets: their gate and up projections are also the first 4096 -> 12288 weights
+    # of the headline rotation
     sets = []
     for _ in range(args.sets):
         g, u, d = (_weights(torch, I, H, gen, dev, torch.float16),
@@ -320,64 +414,14 @@ def main():
                    _weights(torch, H, I, gen, dev, torch.float16))
         sets.append(dict(t=(g, u, d), g=_desc(_lib, *g, I, H), u=_desc(_lib, *u, I, H),
                          d=_desc(_lib, *d, H, I)))
+    keep = [s["t"][0] for s in sets] + [s["t"][1] for s in sets]
+    gate = [s["g"] for s in sets] + [s["u"] for s in sets]
+    while len(gate) < args.weights:
+        b, l = _weights(torch, I, H, gen, dev, torch.float16)
+        keep.append((b, l))
+        gate.append(_desc(_lib, b, l, I, H))
+    gate, keep = gate[:max(args.weights, 1)], keep[:max(args.weights, 1)]
     x = torch.randn(1, H, device=dev, generator=gen).to(act)
-    h = torch.zeros(1, I, dtype=act, device=dev)
-    y = torch.zeros(1, H, dtype=act, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def block(s):
-        st = _lib.lib.flute_mlp_block(ctypes.byref(s["g"]), ctypes.byref(s["u"]),
-                                      ctypes.byref(s["d"]), x.data_ptr(), h.data_ptr(),
-                                      y.data_ptr(), _lib.BF16,
-                                      torch.cuda.current_stream().cuda_stream)
-        if st != 0:
-            raise RuntimeError(_lib.last_error())
-
-    def gate_up(s):
-        st = _lib.lib.flute_gemv_mlp(ctypes.byref(s["g"]), ctypes.byref(s["u"]), x.data_ptr(),
-                                     h.data_ptr(), _lib.BF16, 0,
-                                     torch.cuda.current_stream().cuda_stream)
-        if st != 0:
-            raise RuntimeError(_lib.last_error())
-
-    # ---- parity gate on the first set (a row whose check failed is never reported) ----
-    block(sets[0])
-    torch.cuda.synchronize()
-    sys.path.insert(0, os.path.join(ROOT, "oracle"))
-    import flute_oracle as O
-    (gb, gl), (ub, ul), (db, dl) = sets[0]["t"]
-
-    def oracle_rows(blob, lut, K, tile):
-        # the 128 rows of one tile, dequantised by the oracle from the blob bytes
-        per = (K // 64) * 4096
-        sub = blob[tile * per:(tile + 1) * per].cpu().numpy()
-        return O.dequant(sub, lut[tile:tile + 1].cpu(), 128, K, GS, 4).double()
-
-    xd = x.cpu().double()
-    hd = h.cpu().double()
-    # Beside each error: what rounding the oracle's exact value to the output type costs by
-    # itself (bf16 keeps 8 bits: about 1.1e-3 to 1.6e-3 in relative L2 on these rows), i.e.
-    # the error of a result that is exact before its one rounding.
-    num = den = flo = 0.0
-    for tile in (0, 37, 95):
-        g_ = xd @ oracle_rows(gb, gl, H, tile).t()
-        u_ = xd @ oracle_rows(ub, ul, H, tile).t()
-        ref = O.silu_mul_exact(g_, u_)
-        got = hd[:, tile * 128:(tile + 1) * 128]
-        num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
-        flo += float(((ref.to(act).double() - ref) ** 2).sum())
-    err_h, floor_h = (num / den) ** 0.5, (flo / den) ** 0.5
-    num = den = flo = 0.0
-    for tile in (0, 13, 31):
-        ref = hd @ oracle_rows(db, dl, I, tile).t()
-        got = y.cpu().double()[:, tile * 128:(tile + 1) * 128]
-        num += float(((got - ref) ** 2).sum()); den += float((ref ** 2).sum())
-        flo += float(((ref.to(act).double() - ref) ** 2).sum())
-    err_y, floor_y = (num / den) ** 0.5, (flo / den) ** 0.5
-    parity_ok = err_h < 4e-3 and err_y < 4e-3          # bf16 outputs: rounding alone is 2^-9
-    if not parity_ok:
-        print(f"bench.py: parity gate failed (h {err_h:.2e}, y {err_y:.2e})", file=sys.stderr)
-        return 1
 
     if args.calibrate_copy:
         src = torch.randint(0, 255, (64 << 20,), dtype=torch.uint8, device=dev, generator=gen)
@@ -385,51 +429,46 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
 
-    # ---- timed region 1: whole MLP blocks ------------------------------------------
+    # ---- headline: the GEMV 4096 -> 12288, cold --------------------------------------
+    gv = _Gemv(torch, _lib, ctypes, O, dev, act)
+    y = torch.zeros(1, I, dtype=act, device=dev)
     for i in range(args.warmup):
-        block(sets[i % args.sets])
+        _lib.lib.flute_gemv(ctypes.byref(gate[i % len(gate)]), x.data_ptr(), y.data_ptr(), _lib.BF16, 0,
+                            torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    ms_total = _time_graph(torch, lambda: [block(sets[i % args.sets]) for i in range(args.steps)])
-    ms_step = ms_total / args.steps
-
-    # ---- timed region 2: the dominant kernel alone ----------------------------------
-    ms_gu = _time_graph(torch, lambda: [gate_up(sets[i % args.sets])
-                                        for i in range(args.steps)]) / args.steps
-
-    lut_bytes = (I // GS) * 16 * 2
-    bytes_gate_up = 2 * (I * H // 2 + lut_bytes) + H * 2 + I * 2
-    bytes_down = H * I // 2 + (H // GS) * 16 * 2 + I * 2 + H * 2
-    bytes_step = bytes_gate_up + bytes_down
-    value = bytes_step / (ms_step * 1e-3) / 1e9
-    achieved = bytes_gate_up / (ms_gu * 1e-3) / 1e9
-
-    gemm = None if args.no_gemm else _gemm_section(torch, _lib, ctypes, sets, gen, dev, O)
-    extra = None if args.no_extra else _gemv_section(torch, _lib, ctypes, sets, gen, dev, O)
+    head = gv.run("gemv_4096x12288", gate, keep, I, H, x, launches=args.steps)
+    us = head["us_per_call"]
+    wbytes = I * H // 2 + (I // GS) * 32
+    alg_bytes = wbytes + H * 2 + I * 2
+    value = wbytes / us / 1e3
+    achieved = alg_bytes / us / 1e3
 
     out = {
         "metric": "M=1 LUT-GEMV achieved HBM GB/s (% of peak); M=256 LUT-GEMM TFLOP/s (% MFMA)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_step, 5), "higher_is_better": True,
+        "warmup": args.warmup, "ms_per_step": round(us * 1e-3, 6), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32 accumulate, f16 LUT, bf16 act",
         "data": "synthetic",
-        "config": {"workload": "fused MLP decode M=1: gate+up 4096->12288 (merged, SiLU*mul) + "
-                               "down 12288->4096, idx4, group 128, fp16 LUT, bf16 activations",
-                   "weight_sets": args.sets, "bytes_per_step": bytes_step,
+        "config": {"workload": "M=1 LUT-GEMV, MLP up-projection K=4096 -> N=12288, idx4, group 128, fp16 "
+                               "LUT, bf16 activations, cold weights (rotation through "
+                               f"{len(gate)} weights = {len(gate) * wbytes >> 20} MiB)",
+                   "value_counts": "packed index + LUT bytes", "bytes_per_step": wbytes,
                    "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
-                   "timing": "hipGraph replay, events on the launch stream",
-                   "parity_rel_l2": {"h": err_h, "y": err_y,
-                                     "output_rounding_alone": {"h": floor_h, "y": floor_y},
-                                     "gate": 4e-3}},
+                   "timing": f"hipGraph of {args.steps} launches, median of {REPLAYS} replays, events on "
+                             "the launch stream",
+                   "parity_rel_l2": head["parity_rel_l2"],
+                   "output_rounding_alone": head["output_rounding_alone"], "parity_gate": 4e-3},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_GATE_UP_BYTES,
-                     "kernel": "gemv4_kernel (merged gate+up, SiLU*mul)",
-                     "us_per_launch": round(ms_gu * 1e3, 3),
-                     "algorithmic_bytes_per_launch": bytes_gate_up},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": _traffic_from_profile(),
+                     "kernel": "gemv4_kernel<5, 4, 4, false> (16 rows per workgroup, 768 workgroups)",
+                     "us_per_launch": us, "algorithmic_bytes_per_launch": alg_bytes},
     }
-    if gemm is not None:
-        out["gemm"] = gemm
-    if extra is not None:
-        out["other_m1_configs"] = extra
+    if not args.no_gemm:
+        out["gemm"] = _gemm_section(torch, _lib, ctypes, O, dev, gen, sets)
+    if not args.no_extra:
+        out["mlp_block"] = _mlp_block(torch, _lib, ctypes, O, dev, gen, sets, x, act, 240)
+        out["other_m1_configs"] = _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, x)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = _cpu_baseline(torch)
     print(json.dumps(out))
