@@ -170,4 +170,41 @@ __device__ __forceinline__ uint4 bf16_to_f16_scaled8(uint4 v, int shift) {
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// The same conversion in packed 16-bit integer arithmetic, two values per instruction, for
+// the lean GEMV whose prologue is bound by vector-instruction issue.  The largest magnitude
+// goes to float16's top binade (biased exponent 30; bfloat16's largest mantissa stays below
+// 65504), which leaves 29 normal binades below it: adj = max(emax - 30, 0) is subtracted
+// from every biased exponent and the row sums are scaled back by 2^(adj - 112).  Values
+// more than 29 binades below the largest one are flushed (the one binade at the edge maps
+// to a float16 subnormal of at most the same size): a relative error below 2^-29 of the
+// largest magnitude.  Rows that hold an infinity or a NaN (emax = 255) must take the
+// float route above.
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+
+// Running maximum of the magnitudes (sign cleared) of eight bfloat16 values, per half.
+__device__ __forceinline__ uint32_t bf16_max_mag8(uint32_t m, uint4 v) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    u16x2_t r = __builtin_bit_cast(u16x2_t, m);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        r = __builtin_elementwise_max(r, __builtin_bit_cast(u16x2_t, w[q] & 0x7fff7fffu));
+    return __builtin_bit_cast(uint32_t, r);
+}
+// Largest biased exponent held in a packed pair of magnitudes.
+__device__ __forceinline__ uint32_t bf16_mag_exp(uint32_t m) { return max(m & 0xffffu, m >> 16) >> 7; }
+
+__device__ __forceinline__ uint4 bf16_to_f16_top8(uint4 v, uint32_t adj) {
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    const uint32_t a = adj << 7;
+    const u16x2_t av = __builtin_bit_cast(u16x2_t, a | (a << 16));
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        u16x2_t t = __builtin_bit_cast(u16x2_t, w[q] & 0x7fff7fffu);
+        t = __builtin_elementwise_sub_sat(t, av);   // exponent - adj, flushed below
+        t = t << (unsigned short)3;                 // 8.7 -> 5.10 field positions
+        w[q] = (__builtin_bit_cast(uint32_t, t) & 0x7fff7fffu) | (w[q] & 0x80008000u);
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 }  // namespace flute

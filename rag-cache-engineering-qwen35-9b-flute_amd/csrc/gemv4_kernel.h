@@ -252,35 +252,48 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         write_table(lrow);
         first_units(qrow, q, PF0);
         if (convert) {
-            uint32_t e = 0;
+            uint32_t m = 0;
 #pragma unroll
             for (int i = 0; i < XV; ++i)
-                if (x_piece(i) >= 0) e = max(e, bf16_max_exp8(xv[i]));
-            xshift = bf16_row_shift(wavefront_max(e));
+                if (i < x_loads) m = bf16_max_mag8(m, xv[i]);  // idle lanes hold piece 0 of the slice: harmless
+            const uint32_t emax = wavefront_max(bf16_mag_exp(m));
+            if (emax == 255) {                      // an infinity or a NaN: keep it
 #pragma unroll
-            for (int i = 0; i < XV; ++i) xv[i] = bf16_to_f16_scaled8(xv[i], xshift);
+                for (int i = 0; i < XV; ++i) xv[i] = bf16_to_f16_scaled8(xv[i], 0);
+            } else {
+                const uint32_t adj = emax > 30 ? emax - 30 : 0;
+                xshift = (int)adj - 112;
+#pragma unroll
+                for (int i = 0; i < XV; ++i)
+                    if (i < x_loads) xv[i] = bf16_to_f16_top8(xv[i], adj);
+            }
         }
 #pragma unroll
         for (int i = 0; i < XV; ++i) {
-            const int j = x_piece(i);
+            const int j = i < x_loads ? x_piece(i) : -1;
             if (j >= 0) stage8(j, xv[i]);
         }
     } else if (x_direct) {
         // A long K range: two passes over this wavefront's pieces when a scale is needed
         // (the second one reads them from the cache).
+        uint32_t adj = 0;
+        bool finite = true;                         // uniform
         if (convert) {
-            uint32_t e = 0;
+            uint32_t m = 0;
             for (int i = 0; i < x_loads; ++i) {
                 const int j = x_piece(i);
-                if (j >= 0) e = max(e, bf16_max_exp8(*(const uint4 *)(staged_x + k0 + j)));
+                if (j >= 0) m = bf16_max_mag8(m, *(const uint4 *)(staged_x + k0 + j));
             }
-            xshift = bf16_row_shift(wavefront_max(e));
+            const uint32_t emax = wavefront_max(bf16_mag_exp(m));
+            finite = emax != 255;
+            adj = (finite && emax > 30) ? emax - 30 : 0;
+            if (finite) xshift = (int)adj - 112;
         }
         for (int i = 0; i < x_loads; ++i) {
             const int j = x_piece(i);
             if (j >= 0) {
                 const uint4 v = *(const uint4 *)(staged_x + k0 + j);
-                stage8(j, convert ? bf16_to_f16_scaled8(v, xshift) : v);
+                stage8(j, !convert ? v : finite ? bf16_to_f16_top8(v, adj) : bf16_to_f16_scaled8(v, 0));
             }
         }
         write_table(lrow);
