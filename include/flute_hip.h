@@ -240,7 +240,12 @@ int64_t flute_gemv_lds_bytes(const flute_linear *w, int split);
  * the device.  mode: 0 = GEMV, 1 = GEMM. */
 flute_status flute_validate(const flute_linear *w, int mode);
 
-/* Release the per-device split-K workspaces (also done at process exit). */
+/* Release the per-device split-K workspaces (also done at process exit).
+ * The workspace (partial sums and tickets of a K split, residual coefficients, a pre-rotated
+ * input) is one per device, shared by every stream: a call that uses it is ordered only on
+ * the stream it was given, so two such calls must not overlap on different streams of one
+ * device (upstream's workspace has the same single-stream contract, src/gemv_host.h:31-38).
+ * A call that needs it to grow while its stream is capturing is refused (FLUTE_ERR_INVALID). */
 void flute_release_workspaces(void);
 
 /*
