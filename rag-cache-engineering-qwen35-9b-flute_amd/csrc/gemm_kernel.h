@@ -286,7 +286,7 @@ template <int B, int MB, bool BF16, bool PERM = false>
 __device__ __forceinline__ void half_mma(const uint32_t (&Q)[4 * B], int j, const u4_t (&Aj)[MB],
                                          f4_t (&acc)[MB][8], const uint32_t (&lbase)[4],
                                          int code_shift) {
-    constexpr int AHEAD = 1;                             // pairs of operands in flight
+    constexpr int AHEAD = 2;                             // pairs of operands in flight
     u4_t W[AHEAD + 1][2];
 #pragma unroll
     for (int v = 0; v < AHEAD; ++v) {
