@@ -155,7 +155,14 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
         long wgs = 0;
         for (int i = 0; i < (silu_mul ? 1 : count); ++i) wgs += (long)(segs[i].N / rw) * split;
         long per_cu = (wgs + kNumCU - 1) / kNumCU;
-        if (per_cu > 4) per_cu = 4;
+        // The lean all-4-bit kernel needs the full 32 KB table and is built for three
+        // workgroups per CU; grids of many rounds gain more from it than from a fourth
+        // resident workgroup with a half-size table in the general kernel (4096 -> 248320:
+        // 104 us against 127 us).
+        bool lean = true;
+        for (int i = 0; i < count; ++i)
+            lean &= segs[i].b1 == 4 && (segs[i].b2 == 0 || segs[i].b2 == 4) && segs[i].group_size >= 128;
+        if (per_cu > (lean ? 3 : 4)) per_cu = lean ? 3 : 4;
         if (per_cu < 1) per_cu = 1;
         const long fixed = kc * 2 + 4096;
         budget = 14;
