@@ -83,6 +83,65 @@ __device__ __forceinline__ uint32_t lut_value(const uint32_t (&d)[8], int c) {
     return (c & 1) ? (w >> 16) : (w & 0xffffu);
 }
 
+// Eight consecutive columns of an equal-block rotation held by one lane, block/8 lanes side
+// by side: the stages of length 1, 2, 4 are butterflies between the lane's own values, the
+// longer ones pair it with the lane one bit away (ds_swizzle) as in rotate_blocks_inwave,
+// with the same single rounding per stage, so the result is bit-identical to the standalone
+// rotation; sign, scale 1/sqrt(block) and the rounding to the activation type included.
+template <bool ACT_BF16>
+__device__ __forceinline__ void rotate_piece(uint4 &v, const float (&sg)[8], const float (&sc)[8],
+                                             bool has_awq, float inv, int pair_lanes, int lane) {
+    float f[8];
+    const uint32_t wv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint16_t lo = (uint16_t)(wv[e] & 0xffffu), hi = (uint16_t)(wv[e] >> 16);
+        f[2 * e] = ACT_BF16 ? bf2f(lo) : h2f(lo);
+        f[2 * e + 1] = ACT_BF16 ? bf2f(hi) : h2f(hi);
+    }
+    if (has_awq) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] *= sc[e];
+    }
+#pragma unroll
+    for (int len = 1; len < 8; len <<= 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if ((e & len) == 0) {
+                const float a = f[e], c = f[e | len];
+                f[e] = a + c;
+                f[e | len] = a - c;
+            }
+        }
+    }
+    // and_mask 0x1f, or_mask 0, xor_mask m: lane ^ m inside each half of the wavefront
+#define FLUTE_XOR_STAGE(m)                                                                   \
+    if (pair_lanes > (m)) {                                                                  \
+        const float sgn = (lane & (m)) ? -1.0f : 1.0f;                                       \
+        _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                      \
+            const float other = __int_as_float(__builtin_amdgcn_ds_swizzle(                  \
+                __float_as_int(f[e]), ((m) << 10) | 0x1f));                                  \
+            f[e] = fmaf(f[e], sgn, other);                                                   \
+        }                                                                                    \
+    }
+    FLUTE_XOR_STAGE(1)
+    FLUTE_XOR_STAGE(2)
+    FLUTE_XOR_STAGE(4)
+    FLUTE_XOR_STAGE(8)
+    FLUTE_XOR_STAGE(16)
+#undef FLUTE_XOR_STAGE
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float t = f[e] * sg[e] * inv;
+        if (has_awq) t = t / sc[e];
+        const uint32_t a = ACT_BF16 ? f2bf(t) : f2h(t);   // the standalone kernel's rounding
+        if (e & 1) o[e >> 1] |= a << 16;
+        else o[e >> 1] = a;
+    }
+    v = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 // LPGL = log2(lanes per 64-k tile) = log2(2 * rows per workgroup): 4, 5, 6.
 // NW   = wavefronts per workgroup (4 or 8).
 // PF   = index loads a lane keeps in flight (2 or 4).  The host picks a PF that
@@ -216,7 +275,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     load_lut_row(lut, lrow);
     const uint16_t *staged_x = kp->seg[si0].xsrc ? kp->seg[si0].xsrc : p.x;
     const float *staged_signs = kp->seg[si0].signs, *staged_awq = kp->seg[si0].awq;
-    const bool x_direct = staged_signs == nullptr;  // plain copy
+    const bool x_plain = staged_signs == nullptr;   // plain copy
     uint4 q[PF];
     // bfloat16 activations in front of a float16 LUT: the staged units hold x * 2^-xshift,
     // xshift chosen per wavefront (per workgroup when the input is rotated)
@@ -233,6 +292,13 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     };
     const int x_loads = (my_units + UPL - 1) / UPL;
     const bool x_short = x_loads <= XV;             // uniform
+    // Equal rotation blocks that fit a unit of K (the block-128 form) are transformed by the
+    // wavefront that consumes the unit, in the registers its pieces arrive in: sixteen lanes
+    // hold a block of 128 columns eight to a lane, exactly the arrangement of the butterflies
+    // in rotate_blocks_inwave, so the rotated launch keeps the wavefront-local staging (no
+    // workgroup barrier, operand order) of the plain one.
+    const bool rot_inwave = !x_plain && x_short && p.fht_block >= 16 && p.fht_block <= 64 * GPI;
+    const bool x_direct = x_plain || rot_inwave;    // staged in operand order
     if (x_direct && x_short) {
         // The usual case: activations first, then two index loads, the table (its LUT
         // row arrives through the scalar cache meanwhile), the rest of the loads, and
@@ -243,6 +309,18 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             const int j = x_piece(i);
             xv[i] = *(const uint4 *)(staged_x + k0 + (j >= 0 ? j : 0));
         }
+        // signs and scales of a rotated input travel with the activations, ahead of the index
+        // bytes: waiting for them then does not mean waiting for the index loads
+        float sgv[XV][8], scv[XV][8];
+        if (rot_inwave) {
+#pragma unroll
+            for (int i = 0; i < XV; ++i) {
+                if (i >= x_loads) break;
+                const int j = x_piece(i);
+                load_f8(staged_signs, k0 + (j >= 0 ? j : 0), sgv[i]);
+                if (staged_awq) load_f8(staged_awq, k0 + (j >= 0 ? j : 0), scv[i]);
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int n = 0; n < PF0; ++n) {
@@ -251,6 +329,17 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         }
         write_table(lrow);
         first_units(qrow, q, PF0);
+        if (rot_inwave) {
+            const int nst = 31 - __builtin_clz((unsigned)p.fht_block);
+            const float inv = inv_sqrt_pow2(nst);
+            const int pair_lanes = p.fht_block >> 3;    // lanes of one block: 2 .. 32
+#pragma unroll
+            for (int i = 0; i < XV; ++i) {
+                if (i >= x_loads) break;
+                if (p.act_bf16) rotate_piece<true>(xv[i], sgv[i], scv[i], staged_awq != nullptr, inv, pair_lanes, L);
+                else rotate_piece<false>(xv[i], sgv[i], scv[i], staged_awq != nullptr, inv, pair_lanes, L);
+            }
+        }
         if (convert) {
             uint32_t m = 0;
 #pragma unroll
@@ -273,7 +362,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             const int j = i < x_loads ? x_piece(i) : -1;
             if (j >= 0) stage8(j, xv[i]);
         }
-    } else if (x_direct) {
+    } else if (x_plain) {
         // A long K range: two passes over this wavefront's pieces when a scale is needed
         // (the second one reads them from the cache).
         uint32_t adj = 0;
