@@ -439,15 +439,6 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 
         // ---- K loop -----------------------------------------------------------------
         // One step = two 16-byte loads of this lane = 32 lookups and 8 matrix products.
-        auto lookups = [&](const uint4 &qv, uint32_t (&e)[16]) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const uint32_t wv = v == 0 ? qv.x : v == 1 ? qv.y : v == 2 ? qv.z : qv.w;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)         // byte j: d = j >> 1, s2 = j & 1
-                    e[v * 4 + j] = *(LdsWord)((((wv >> (8 * j)) & 0xffu) << ES) + slot);
-            }
-        };
         auto operand_b = [&](int m0, int m1) -> gv_u4_t {
             const int u0 = w + m0 * NW, u1 = w + m1 * NW;
             if (x_direct) {
@@ -457,58 +448,55 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             const int a0 = u0 * (32 * GPI) + xnat, a1 = u1 * (32 * GPI) + xnat;
             return (gv_u4_t){xs32[a0], xs32[a0 + 4], xs32[a1], xs32[a1 + 4]};
         };
-        auto products = [&](const uint32_t (&e0)[16], const uint32_t (&e1)[16], gv_u4_t B) {
+        // two units (two 16-byte loads of this lane): per row group v, eight lookups feed two
+        // matrix products
+        auto unit_pair = [&](const uint4 &qa, const uint4 &qb, gv_u4_t B) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t wa = v == 0 ? qa.x : v == 1 ? qa.y : v == 2 ? qa.z : qa.w;
+                const uint32_t wb = v == 0 ? qb.x : v == 1 ? qb.y : v == 2 ? qb.z : qb.w;
+                uint32_t e[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {       // byte j: d = j >> 1, s2 = j & 1
+                    e[j] = *(LdsWord)((((wa >> (8 * j)) & 0xffu) << ES) + slot);
+                    e[4 + j] = *(LdsWord)((((wb >> (8 * j)) & 0xffu) << ES) + slot);
+                }
 #pragma unroll
                 for (int d = 0; d < 2; ++d) {
-                    const gv_u4_t A = {e0[v * 4 + 2 * d], e0[v * 4 + 2 * d + 1], e1[v * 4 + 2 * d],
-                                       e1[v * 4 + 2 * d + 1]};
+                    const gv_u4_t A = {e[2 * d], e[2 * d + 1], e[4 + 2 * d], e[4 + 2 * d + 1]};
                     acc[v * 2 + d] = gv_mfma<BF16>(A, B, acc[v * 2 + d]);
                 }
+            }
         };
         int nb = 0;
         __builtin_amdgcn_s_setprio(2);
         for (; nb + 2 * PF <= my_units; nb += PF) {          // every refill exists
 #pragma unroll
             for (int n = 0; n < PF; n += 2) {
-                uint32_t e0[16], e1[16];
                 const gv_u4_t B = operand_b(nb + n, nb + n + 1);
-                lookups(q[n], e0);
-                lookups(q[n + 1], e1);
-                // pinned: the scheduler would otherwise sink all refills to the end of
-                // the body, draining the prefetch queue once per group
+                unit_pair(q[n], q[n + 1], B);
                 __builtin_amdgcn_sched_barrier(0);
                 q[n] = load_idx16(qrow + (size_t)(nb + n + PF) * step + lane0);
                 q[n + 1] = load_idx16(qrow + (size_t)(nb + n + 1 + PF) * step + lane0);
                 __builtin_amdgcn_sched_barrier(0);
-                products(e0, e1, B);
             }
         }
         if (!has_next) __builtin_amdgcn_s_setprio(1);
-        // the last group (my_units is a multiple of PF), refilled from the next pass when
-        // there is one; two copies so that the loads of each are unconditional
         if (has_next) {
 #pragma unroll
             for (int n = 0; n < PF; n += 2) {
-                uint32_t e0[16], e1[16];
                 const gv_u4_t B = operand_b(nb + n, nb + n + 1);
-                lookups(q[n], e0);
-                lookups(q[n + 1], e1);
+                unit_pair(q[n], q[n + 1], B);
                 __builtin_amdgcn_sched_barrier(0);
                 q[n] = load_idx16(qnext + (size_t)n * step + lane0);
                 q[n + 1] = load_idx16(qnext + (size_t)(n + 1) * step + lane0);
                 __builtin_amdgcn_sched_barrier(0);
-                products(e0, e1, B);
             }
         } else {
 #pragma unroll
             for (int n = 0; n < PF; n += 2) {
-                uint32_t e0[16], e1[16];
                 const gv_u4_t B = operand_b(nb + n, nb + n + 1);
-                lookups(q[n], e0);
-                lookups(q[n + 1], e1);
-                products(e0, e1, B);
+                unit_pair(q[n], q[n + 1], B);
             }
         }
 
