@@ -593,3 +593,41 @@ def embedding_gather(ids, indices, lut, N: int, K: int, bitwidth: int, group_siz
                                   _stream_of(A)))
     del keep
     return out.reshape(*ids.shape, int(K))
+
+
+# ---------------------------------------------------------------------------
+# compiled binding
+# ---------------------------------------------------------------------------
+# flute_extended/_C_native (csrc/torch_binding.cpp, built by csrc/build_torch_binding.py) is
+# the compiled PyTorch-ROCm counterpart of upstream's pybind module for the entries a decode
+# loop calls per token.  When it is built and speaks this library's ABI it takes those names
+# over (same signatures, checks and messages; about a third of the host time per call); the
+# Python forms above stay reachable as PYTHON_BINDING[name], serve everything else, and serve
+# all of it when the module is absent or FLUTE_PYTHON_BINDING is set.  Either way the
+# kernels are the ones in libflute_hip.so: there is no other implementation to fall back to.
+
+NATIVE_NAMES = ("qgemm_gemv_stream", "qgemm_gemv_fht_stream", "qgemm_gemv_splitk_stream",
+                "qgemm_gemv_splitk_fht_stream", "qgemm_gemv_multi", "qgemm_gemv_mlp",
+                "qgemm_cutlass_streaming", "qgemm_dual_stream")
+PYTHON_BINDING = {name: globals()[name] for name in NATIVE_NAMES}
+native = None
+
+
+def _load_native():
+    import os
+    if os.environ.get("FLUTE_PYTHON_BINDING"):
+        return None
+    try:
+        from . import _C_native
+    except ImportError:
+        return None
+    if _C_native.abi_version() != lib.flute_abi_version():
+        return None
+    return _C_native
+
+
+native = _load_native()
+if native is not None:
+    for _name in NATIVE_NAMES:
+        globals()[_name] = getattr(native, _name)
+    del _name

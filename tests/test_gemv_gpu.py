@@ -15,6 +15,7 @@ import torch
 import flute_extended as fx
 import flute_oracle as O
 from _util import make_weight, make_x, rel_l2
+from flute_extended import _C
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -299,3 +300,44 @@ def test_merged_gate_up_with_activations_beyond_the_float16_range():
     ref = O.silu_mul_exact(yg, yu).to(torch.bfloat16)
     assert torch.isfinite(out).all()
     assert rel_l2(out.cpu(), ref) <= 4e-3       # one bfloat16 rounding of a product of two sums
+
+
+@pytest.mark.skipif(_C.native is None, reason="the compiled binding is not built or switched off")
+def test_compiled_binding_gives_the_python_binding_s_outputs():
+    """flute_extended._C_native (csrc/torch_binding.cpp, the counterpart of upstream's pybind
+    module, src/bindings.cpp:230-546) and the ctypes mirror call the same kernels with the same
+    descriptor: outputs agree bit for bit, for a GEMV with every optional operand, a grouped and
+    a merged launch, and both GEMM entries."""
+    N, K = 512, 1024
+    w = make_weight(N, K, 4, 128, seed=5, bits2=1, rank=8, bias=True, device=DEV)
+    x = make_x(1, K, seed=6).to(DEV)
+    signs = O.rotation_signs(K, 1).to(DEV)
+    e32 = torch.empty(0, dtype=torch.float32, device=DEV)
+    args = (x, w["blob_d"], w["lut_d"], 4, w["blob2_d"], w["lut2_d"], 1, w["resB_d"], w["resA_d"],
+            w["bias_d"], 128)
+    for name, extra in (("qgemm_gemv_splitk_stream", (2,)), ("qgemm_gemv_splitk_fht_stream", (signs, e32, 1, 128)),
+                        ("qgemm_gemv_fht_stream", (signs, e32))):
+        a = _C.PYTHON_BINDING[name](*args, *extra)
+        b = getattr(_C.native, name)(*args, *extra)
+        assert torch.equal(a, b), name
+    xm = make_x(9, K, seed=7).to(DEV)
+    argm = (xm,) + args[1:]
+    assert torch.equal(_C.PYTHON_BINDING["qgemm_dual_stream"](*argm), _C.native.qgemm_dual_stream(*argm))
+    assert torch.equal(_C.PYTHON_BINDING["qgemm_cutlass_streaming"](xm, w["blob_d"], w["lut_d"], 4, 128),
+                       _C.native.qgemm_cutlass_streaming(xm, w["blob_d"], w["lut_d"], 4, 128))
+    # segment table: gate/up of a merged launch, then the same two weights as a grouped launch
+    u = make_weight(N, K, 4, 128, seed=8, device=DEV)
+    outs = [torch.zeros(1, N, dtype=torch.float16, device=DEV) for _ in range(6)]
+    def table(c0, c1):
+        rows = []
+        for t, c in ((w, c0), (u, c1)):
+            rows.append([t["blob_d"].data_ptr(), t["lut_d"].data_ptr(), 0, 0, 0, 0, 0, c.data_ptr(),
+                         N, 0, 4, 0, 128, 0, 0])
+        return torch.tensor(rows, dtype=torch.int64)
+    _C.PYTHON_BINDING["qgemm_gemv_multi"](x, table(outs[0], outs[1]))
+    _C.native.qgemm_gemv_multi(x, table(outs[2], outs[3]))
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[3])
+    _C.PYTHON_BINDING["qgemm_gemv_mlp"](x, table(outs[0], outs[1]), outs[4])
+    _C.native.qgemm_gemv_mlp(x, table(outs[0], outs[1]), outs[5])
+    torch.cuda.synchronize()
+    assert torch.equal(outs[4], outs[5]) and outs[4].abs().sum() > 0

@@ -134,6 +134,46 @@ def test_tensor_level_refusals_raise_runtimeerror():
         fx.qgemm_gemv_stream(x, w["blob"], w["lut"], 4, 32)         # plain entry: gs >= 64 only
 
 
+def _first_line(fn):
+    with pytest.raises(RuntimeError) as err:
+        fn()
+    return str(err.value).splitlines()[0]
+
+
+@pytest.mark.skipif(_C.native is None, reason="the compiled binding is not built or switched off")
+def test_compiled_binding_refuses_with_the_python_binding_s_words():
+    """csrc/torch_binding.cpp restates the checks of flute_extended/_C.py (upstream: the
+    TORCH_CHECKs of src/kernel_gemv.cu:338-454): same order, same first line."""
+    x, w = _cpu_args()
+    e8 = torch.empty(0, dtype=torch.uint8)
+    e16 = torch.empty(0, dtype=torch.float16)
+    base = dict(A=x, indices=w["blob"], lut=w["lut"], b1=4, i2=e8, l2=e16, b2=0, rb=e16, ra=e16,
+                bi=e16, gs=128)
+    cases = [dict(), dict(A=make_x(2, 128)), dict(A=make_x(1, 96)), dict(A=make_x(1, 128, dtype=torch.float32)),
+             dict(indices=w["blob"][:-7]), dict(lut=w["lut"][:, :8].contiguous()), dict(gs=48),
+             dict(b1=5), dict(b2=7), dict(rb=torch.zeros(4, 128, dtype=torch.float16)),
+             dict(rb=torch.zeros(300, 128, dtype=torch.float16), ra=torch.zeros(256, 300, dtype=torch.float16)),
+             dict(bi=torch.zeros(7, dtype=torch.float16)),
+             dict(b2=1, i2=torch.zeros(3, dtype=torch.uint8), l2=torch.zeros(2, 2, dtype=torch.float16)),
+             dict(lut=w["lut"].bfloat16())]
+    for name in ("qgemm_gemv_splitk_stream", "qgemm_dual_stream"):
+        for over in cases:
+            a = dict(base, **over)
+            args = (a["A"], a["indices"], a["lut"], a["b1"], a["i2"], a["l2"], a["b2"], a["rb"],
+                    a["ra"], a["bi"], a["gs"])
+            if name == "qgemm_dual_stream" and "A" in over and over["A"].shape[0] == 2:
+                continue                                   # M = 2 is fine for the GEMM
+            py = _first_line(lambda: _C.PYTHON_BINDING[name](*args))
+            cc = _first_line(lambda: getattr(_C.native, name)(*args))
+            assert py == cc, (name, over.keys(), py, cc)
+    seg = torch.zeros(2, 15, dtype=torch.int64)
+    for args in ((x, seg[:, :14].contiguous(), e16), (make_x(2, 128), seg, e16),
+                 (x, seg, torch.zeros(5, dtype=torch.float32))):
+        py = _first_line(lambda: _C.PYTHON_BINDING["qgemm_gemv_mlp"](*args))
+        cc = _first_line(lambda: _C.native.qgemm_gemv_mlp(*args))
+        assert py == cc
+
+
 def test_layout_string_guards():
     x, w = _cpu_args()
     with pytest.raises(ValueError):
