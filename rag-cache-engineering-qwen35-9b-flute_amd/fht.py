@@ -121,38 +121,44 @@ def _butterfly(v: torch.Tensor) -> torch.Tensor:
 
 
 def _check(x: torch.Tensor, signs: torch.Tensor) -> Tuple[int, int]:
-    if signs.dim() != 1 or signs.numel() != x.shape[-1]:
+    """(rows, K) of x seen as a matrix over its last axis; refuses what upstream refuses
+    (fht.py:195-203 upstream), with its exception types."""
+    K = int(x.shape[-1]) if x.dim() > 0 else 0
+    if not x.is_floating_point():
+        raise TypeError(f"fht: x must be floating point, got {x.dtype}")
+    if K < 1:
+        raise ValueError("fht: x's last dim must be >= 1")
+    if tuple(signs.shape) != (K,):
         raise ValueError(f"fht: signs must be a (K,) vector matching x's last dim "
                          f"(got signs {tuple(signs.shape)}, x {tuple(x.shape)})")
-    if not torch.is_floating_point(x):
-        raise TypeError(f"fht: x must be floating point, got {x.dtype}")
-    if x.shape[-1] < 1:
-        raise ValueError("fht: x's last dim must be >= 1")
-    return x.numel() // x.shape[-1], int(x.shape[-1])
+    return x.numel() // K, K
+
+
+def _per_segment(x: torch.Tensor, signs: torch.Tensor, signs_first: bool) -> torch.Tensor:
+    """The torch transform both directions share: every segment of the last axis goes through
+    the butterfly in fp32 and is scaled by 1/sqrt(its width); the signs multiply the output
+    (forward, x @ T) or the input (adjoint, v @ T^T).  fht.py:206-238 upstream."""
+    rows, K = _check(x, signs)
+    widths = [b for _, b in segments(K)]
+    flat = x.reshape(rows, K).to(torch.float32)
+    sgn = signs.to(device=flat.device, dtype=torch.float32)
+    pieces = []
+    for part, sg in zip(torch.split(flat, widths, dim=1), torch.split(sgn, widths)):
+        part = part * sg if signs_first else part
+        part = _butterfly(part.contiguous())
+        part = part if signs_first else part * sg
+        pieces.append(part * (1.0 / math.sqrt(part.shape[1])))
+    return torch.cat(pieces, dim=1).reshape(x.shape).to(x.dtype)
 
 
 def fht_reference(x: torch.Tensor, signs: torch.Tensor) -> torch.Tensor:
     """((x @ H) * s) * (1/sqrt(b)) per segment, fp32, returned in x's dtype."""
-    M, K = _check(x, signs)
-    v = x.reshape(M, K).float()
-    s = signs.to(v.device).float().view(1, K)
-    out = torch.empty_like(v)
-    for off, b in segments(K):
-        seg = _butterfly(v[:, off:off + b].contiguous())
-        out[:, off:off + b] = (seg * s[:, off:off + b]) * (1.0 / math.sqrt(b))
-    return out.reshape(x.shape).to(x.dtype)
+    return _per_segment(x, signs, signs_first=False)
 
 
 def fht_reference_adjoint(v: torch.Tensor, signs: torch.Tensor) -> torch.Tensor:
     """((v * s) @ H) * (1/sqrt(b)) per segment."""
-    M, K = _check(v, signs)
-    g = v.reshape(M, K).float()
-    s = signs.to(g.device).float().view(1, K)
-    out = torch.empty_like(g)
-    for off, b in segments(K):
-        seg = _butterfly((g[:, off:off + b] * s[:, off:off + b]).contiguous())
-        out[:, off:off + b] = seg * (1.0 / math.sqrt(b))
-    return out.reshape(v.shape).to(v.dtype)
+    return _per_segment(v, signs, signs_first=True)
 
 
 def fht_matmul(x: torch.Tensor, signs: torch.Tensor, K: Optional[int] = None,
