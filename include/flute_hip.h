@@ -242,9 +242,11 @@ flute_status flute_validate(const flute_linear *w, int mode);
 
 /* Release the per-device split-K workspaces (also done at process exit).
  * The workspace (partial sums and tickets of a K split, residual coefficients, a pre-rotated
- * input) is one per device, shared by every stream: a call that uses it is ordered only on
- * the stream it was given, so two such calls must not overlap on different streams of one
- * device (upstream's workspace has the same single-stream contract, src/gemv_host.h:31-38).
+ * input, the GEMM's operand image) is one per device, shared by every stream (upstream's
+ * has a single-stream contract, src/gemv_host.h:31-38).  A call on another stream than the
+ * previous user's is ordered behind it with an event, so eager work on two streams stays
+ * correct (and serialised); what remains the caller's to order: calls issued at the same
+ * moment from two host threads, and streams under capture (no event is inserted there).
  * A call that needs it to grow while its stream is capturing is refused (FLUTE_ERR_INVALID). */
 void flute_release_workspaces(void);
 

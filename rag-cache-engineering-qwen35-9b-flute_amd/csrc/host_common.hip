@@ -85,6 +85,11 @@ struct Workspace {
     int *tickets = nullptr;
     size_t floats = 0;
     size_t ints = 0;
+    // the stream of the last call that took the workspace, and an event to order the next
+    // stream behind it
+    hipStream_t last_stream = nullptr;
+    bool used = false;
+    hipEvent_t handover = nullptr;
 };
 
 static std::mutex g_ws_mu;
@@ -140,6 +145,29 @@ flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float
         ws.tickets = fresh;
         ws.ints = want;
     }
+    // One workspace serves every stream of the device.  A call on another stream than the last
+    // one is ordered behind it with an event, so that two eager streams cannot overwrite each
+    // other's partial sums; calls that really overlap (issued from two host threads at once)
+    // and streams under capture (an event of a foreign stream cannot join a capture) remain
+    // the caller's to order.
+    if (ws.used && ws.last_stream != stream) {
+        hipStreamCaptureStatus mine = hipStreamCaptureStatusNone, theirs = hipStreamCaptureStatusNone;
+        FLUTE_HIP_CHECK(hipStreamIsCapturing(stream, &mine));
+        // the earlier stream may be gone by now (its work is then complete): a failing query
+        // means there is nothing to wait for
+        const bool alive = hipStreamIsCapturing(ws.last_stream, &theirs) == hipSuccess;
+        if (!alive) (void)hipGetLastError();
+        if (alive && mine == hipStreamCaptureStatusNone && theirs == hipStreamCaptureStatusNone) {
+            if (!ws.handover)
+                FLUTE_HIP_CHECK(hipEventCreateWithFlags(&ws.handover, hipEventDisableTiming));
+            if (hipEventRecord(ws.handover, ws.last_stream) == hipSuccess)
+                FLUTE_HIP_CHECK(hipStreamWaitEvent(stream, ws.handover, 0));
+            else
+                (void)hipGetLastError();
+        }
+    }
+    ws.last_stream = stream;
+    ws.used = true;
     *P = ws.P;
     *tickets = ws.tickets;
     return FLUTE_OK;
@@ -213,6 +241,7 @@ void flute_release_workspaces(void) {
     for (auto &kv : flute::g_ws) {
         if (kv.second.P) (void)hipFree(kv.second.P);
         if (kv.second.tickets) (void)hipFree(kv.second.tickets);
+        if (kv.second.handover) (void)hipEventDestroy(kv.second.handover);
     }
     flute::g_ws.clear();
     for (void *p : flute::g_retired) (void)hipFree(p);

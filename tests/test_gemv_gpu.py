@@ -302,6 +302,26 @@ def test_merged_gate_up_with_activations_beyond_the_float16_range():
     assert rel_l2(out.cpu(), ref) <= 4e-3       # one bfloat16 rounding of a product of two sums
 
 
+def test_two_streams_share_the_workspace_in_order():
+    """The split-K workspace is one per device (upstream: one stream only,
+    src/gemv_host.h:31-38).  Launches that alternate between two streams, with nothing but the
+    library's own hand-over between them, must still give the single-stream result."""
+    N, K = 256, 8192
+    ws = [make_weight(N, K, 4, 128, seed=40 + i, rank=8, device=DEV) for i in range(2)]
+    x = make_x(1, K, seed=9).to(DEV)
+    want = [_run(w, x, split=8).cpu() for w in ws]
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    got = []
+    for rep in range(20):
+        for st, w in ((s1, ws[0]), (s2, ws[1])):
+            with torch.cuda.stream(st):
+                got.append((rep, _run(w, x, split=8)))
+    torch.cuda.synchronize()
+    for i, (rep, y) in enumerate(got):
+        assert torch.equal(y.cpu(), want[i % 2]), (rep, i % 2)
+
+
 @pytest.mark.skipif(_C.native is None, reason="the compiled binding is not built or switched off")
 def test_compiled_binding_gives_the_python_binding_s_outputs():
     """flute_extended._C_native (csrc/torch_binding.cpp, the counterpart of upstream's pybind
