@@ -211,6 +211,25 @@ def test_fused_block_rotation_is_bit_identical_to_rotate_then_gemv(block, dtype)
     assert rel_l2(fused.cpu(), _exact(w, xo).to(dtype)) <= (TOL if dtype == torch.float16 else 4e-3)
 
 
+@pytest.mark.parametrize("N,block", [(512, 64), (512, 128), (4096, 128), (4096, 64), (1024, 256)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_block_rotation_with_scale_compensation_matches_the_chain(N, block, dtype):
+    """((x * s) @ T_block) / s in the GEMV prologue (fht.py:207-238 upstream for the transform)
+    against the rotation kernel followed by the plain GEMV, bit for bit; the shapes cover
+    rotation in the consuming wavefront's registers (a block fits a unit of K) and the
+    staged form (it does not)."""
+    from flute_extended import _C
+    K = 4096
+    w = make_weight(N, K, 4, 128, seed=block + N, act_dtype=dtype, device=DEV)
+    x = make_x(1, K, seed=13, dtype=dtype)
+    signs = O.rotation_signs(K, block + 1)
+    g = torch.Generator().manual_seed(block)
+    s = (torch.rand(K, generator=g) * 1.5 + 0.5).float()
+    fused = _run(w, x, signs=signs, awq=s, rot_block=block)
+    xr = _C._fht("chain", x.to(DEV), signs.to(DEV), s.to(DEV), None, 0, block)
+    assert torch.equal(fused, _run(w, xr.cpu()))
+
+
 def test_workspace_growth_is_refused_under_graph_capture():
     """A K split needs the library workspace.  When that would have to be allocated while
     the stream is being captured, the call is refused (an allocation and the clearing of
