@@ -224,11 +224,12 @@ flute_status flute_embedding(const flute_linear *w, const int64_t *ids, int64_t 
                              void *out, void *stream);
 
 /*
- * The K-split the library would choose for an (N, K) GEMV on this device
- * (the MI355X counterpart of gemv_pick_split, src/gemv_host.cpp:29-38).  On this
- * device the unsplit launch measured fastest for every shape, so the answer is 1;
- * callers that pass an explicit split to flute_gemv still get it.
- * Pure host arithmetic: usable without a GPU.
+ * The K-split the library would choose for an (N, K) GEMV without a fused rotation on this
+ * device (the MI355X counterpart of gemv_pick_split, src/gemv_host.cpp:29-38; the numbers
+ * are this device's, not the A10G's).  Up to K = 24576 the unsplit launch measured fastest
+ * for every N, so the answer is 1; from K = 32768 it is 4 for N <= 512 and 2 for N <= 1024
+ * (N = 512, K = 32768: 7.5 us against 9.0 us unsplit).  Callers that pass an explicit split
+ * to flute_gemv still get it.  Pure host arithmetic: usable without a GPU.
  */
 int flute_pick_split(int N, int K);
 

@@ -41,13 +41,18 @@ struct Plan {
 };
 
 // Shape of the launch for `rows` output rows over G tiles of K.  A workgroup
-// owns `rw` rows.  The library's own policy never splits K: the exchange between
-// workgroups (partial sums written through, a ticket, the last arrival reading them
-// back) is three memory round trips, about 1.5 us, and measured slower than the
-// unsplit launch with eight wavefronts for every narrow shape tried (N = 128...3072
-// at K = 2048...16384; e.g. N = 1024, K = 4096: 5.0 us against 6.7 us split four
-// ways).  A caller's explicit split is honoured.
-void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *waves) {
+// owns `rw` rows.  The library's own policy splits K only where a workgroup's K range
+// would be very long over few rows: the exchange between workgroups (partial sums
+// written through, a ticket, the last arrival reading them back) is three memory round
+// trips, and up to K = 24576 the unsplit launch measured faster for every narrow shape
+// (N = 128...3072; e.g. N = 1024, K = 4096: 4.5 us against 5.9 / 10.4 / 11.4 us split
+// 2 / 4 / 8 ways; N = 512, K = 24576: 7.7 against 8.2 / 11.5).  From K = 32768 on, four
+// ways win up to 512 rows and two ways up to 1024 (K = 32768: N = 128 6.8 against
+// 8.7 us, N = 512 7.5 against 9.0, N = 1024 8.3 against 9.2; K = 65536: N = 512 8.8
+// against 19.0, N = 1024 12.8 against 20.9); 2048 rows and more stay unsplit (11.0
+// against 14.3 us).  A caller's explicit split is honoured.
+void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *waves,
+                  bool may_split = true) {
     int best_rw = tuning().gemv_rw;
     if (best_rw != 8 && best_rw != 16 && best_rw != 32) {
         // The narrowest slices whose grid is still resident at once (three four-wavefront
@@ -73,6 +78,9 @@ void choose_shape(int rows, int G, int split_req, int *rw, int *split, int *wave
         while (G % sp == 0 && (G / sp) % (32 / best_rw) != 0 && best_rw < 32) best_rw *= 2;
     } else {
         sp = 1;
+        // (not with a rotation fused into the prologue: its blocks would have to fit the slices)
+        if (may_split && G >= 512 && rows <= 512 && G % 4 == 0) sp = 4;
+        else if (may_split && G >= 512 && rows <= 1024 && G % 2 == 0) sp = 2;
         while ((G / sp) % (32 / best_rw) != 0 && best_rw < 32) best_rw *= 2;
     }
     *rw = best_rw;
@@ -133,7 +141,9 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     int rows = 0;
     for (int i = 0; i < (silu_mul ? 1 : count); ++i) rows += segs[i].N;
     int rw, waves;
-    choose_shape(rows, G, split, &rw, &split, &waves);
+    bool rotated = false;
+    for (int i = 0; i < count; ++i) rotated |= segs[i].signs != nullptr;
+    choose_shape(rows, G, split, &rw, &split, &waves, !rotated);
     FLUTE_REQUIRE((G / split) % (32 / rw) == 0, FLUTE_ERR_UNSUPPORTED,
                   "%s: K/64/split = %d is not a whole number of wavefront loads", who, G / split);
     const int gs_tiles = G / split;

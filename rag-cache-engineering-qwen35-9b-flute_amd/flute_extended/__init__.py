@@ -256,10 +256,12 @@ GEMV_SPLITK_MAX_RESIDUAL_RANK = 256
 def gemv_split_hint(N: int, K: int) -> int:
     """The K split the library picks for an (N, K) single-stream GEMV on this
     device.  Upstream's policy targets 160 workgroups on 80 SMs
-    (src/gemv_host.cpp:29-38).  On the MI355X the unsplit launch measured fastest for
-    every shape (N = 1024, K = 4096: 4.8 us against 6.0 / 10.0 / 11.1 us split 2 / 4 / 8
-    ways: the exchange of partial sums costs three memory round trips), so the answer is
-    1; an explicit split passed to the split-K entry points is still honoured."""
+    (src/gemv_host.cpp:29-38).  On the MI355X the unsplit launch measured fastest up to
+    K = 24576 for every N (N = 1024, K = 4096: 4.5 us against 5.9 / 10.4 / 11.4 us split
+    2 / 4 / 8 ways: the exchange of partial sums costs three memory round trips), so the
+    answer is 1 there; from K = 32768 it is 4 for N <= 512 and 2 for N <= 1024 (N = 512,
+    K = 32768: 7.5 us against 9.0 us unsplit).  An explicit split passed to the split-K
+    entry points is always honoured."""
     return _C.pick_split(int(N), int(K))
 
 

@@ -321,6 +321,19 @@ def test_merged_gate_up_with_activations_beyond_the_float16_range():
     assert rel_l2(out.cpu(), ref) <= 4e-3       # one bfloat16 rounding of a product of two sums
 
 
+def test_long_k_narrow_output_takes_the_library_s_split():
+    """K = 32768 over 256 rows: the library's own choice is a four-way K split
+    (upstream's policy: src/gemv_host.cpp:29-38); the result is the forced four-way
+    split bit for bit, deterministic, and within tolerance of the oracle."""
+    N, K = 256, 32768
+    assert fx.gemv_split_hint(N, K) == 4
+    w = make_weight(N, K, 4, 128, seed=77, device=DEV)
+    x = make_x(1, K, seed=78)
+    y = _run(w, x)
+    assert torch.equal(y, _run(w, x, split=4)) and torch.equal(y, _run(w, x))
+    assert rel_l2(y.cpu(), _exact(w, x).half()) <= TOL
+
+
 def test_two_streams_share_the_workspace_in_order():
     """The split-K workspace is one per device (upstream: one stream only,
     src/gemv_host.h:31-38).  Launches that alternate between two streams, with nothing but the

@@ -211,12 +211,17 @@ def test_gates_and_tables():
     assert fx.gemv_multi_supported(4096, 48, [(4, 0, 128), (3, 3, 64)])
     assert fx.dual_stream_supported(4, 0, 128, 4096, 4096)
     assert not fx.dual_stream_supported(4, 0, 128, 4000, 4096)
-    # the split policy of this library: a hint always divides K/64 (on this device the
-    # unsplit launch measured fastest for wide and narrow outputs alike, so the hint is 1)
+    # the split policy of this library (upstream's: src/gemv_host.cpp:29-38, other numbers): a
+    # hint always divides K/64; the unsplit launch measured fastest up to K = 24576, from
+    # K = 32768 narrow outputs split four ways (N <= 512) or two ways (N <= 1024)
     assert fx.gemv_split_hint(12288, 4096) == 1 and fx.gemv_split_hint(248320, 4096) == 1
     for N in (1024, 512, 128):
         s = fx.gemv_split_hint(N, 4096)
         assert s >= 1 and 64 % s == 0
+        assert fx.gemv_split_hint(N, 24576) == 1
+    assert fx.gemv_split_hint(512, 32768) == 4 and fx.gemv_split_hint(128, 65536) == 4
+    assert fx.gemv_split_hint(1024, 32768) == 2 and fx.gemv_split_hint(2048, 32768) == 1
+    assert fx.gemv_split_hint(512, 32768 + 64) == 1          # 513 tiles: neither 4 nor 2 divides
     assert 0 < _C.gemv_lds_bytes(12288, 4096, 4, 0, 128) <= fx.LDS_BYTES_PER_CU
 
 
