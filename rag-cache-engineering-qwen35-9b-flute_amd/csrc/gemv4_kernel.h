@@ -206,6 +206,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // the dynamic LDS block is folded into the per-lane replica offset once.
     typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    // The kernel has no static LDS, so its dynamic block starts at address 0 and a lane's slot
+    // stays below the table stride: (code << 7) and the slot share no bits, which lets the
+    // address of byte 0 be formed as shift + and-or, two instructions like the other bytes.
+    __builtin_assume(lds_base == 0);
     const uint32_t slot = lds_base + (uint32_t)(L & 31) * 4u;
     const int e_own = tid & 255;                    // table entry this thread writes
     const int share = tid >> 8;
@@ -455,17 +459,16 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             for (int v = 0; v < 4; ++v) {
                 const uint32_t wa = v == 0 ? qa.x : v == 1 ? qa.y : v == 2 ? qa.z : qa.w;
                 const uint32_t wb = v == 0 ? qb.x : v == 1 ? qb.y : v == 2 ? qb.z : qb.w;
-                uint32_t e[8];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {       // byte j: d = j >> 1, s2 = j & 1
-                    e[j] = *(LdsWord)((((wa >> (8 * j)) & 0xffu) << ES) + slot);
-                    e[4 + j] = *(LdsWord)((((wb >> (8 * j)) & 0xffu) << ES) + slot);
-                }
-#pragma unroll
-                for (int d = 0; d < 2; ++d) {
-                    const gv_u4_t A = {e[2 * d], e[2 * d + 1], e[4 + 2 * d], e[4 + 2 * d + 1]};
-                    acc[v * 2 + d] = gv_mfma<BF16>(A, B, acc[v * 2 + d]);
-                }
+                // byte j of a dword: d = j >> 1, s2 = j & 1; an operand is (s2 = 0, 1) of both units
+                auto look = [&](uint32_t wq, int j) -> uint32_t {
+                    // byte 0: shift, then one and-or (the slot lies below the stride)
+                    if (j == 0) return *(LdsWord)(((wq << ES) & (0xffu << ES)) | slot);
+                    return *(LdsWord)((((wq >> (8 * j)) & 0xffu) << ES) + slot);
+                };
+                const gv_u4_t A0 = {look(wa, 0), look(wa, 1), look(wb, 0), look(wb, 1)};
+                const gv_u4_t A1 = {look(wa, 2), look(wa, 3), look(wb, 2), look(wb, 3)};
+                acc[v * 2] = gv_mfma<BF16>(A0, B, acc[v * 2]);
+                acc[v * 2 + 1] = gv_mfma<BF16>(A1, B, acc[v * 2 + 1]);
             }
         };
         int nb = 0;
