@@ -254,8 +254,9 @@ void flute_release_workspaces(void);
 /*
  * The launchers read their tuning and test knobs (FLUTE_GEMV_RW, FLUTE_GEMV_WAVES,
  * FLUTE_GEMV_TABLE_LOG2, FLUTE_GEMV_PREROTATE, FLUTE_GEMV4_PF, FLUTE_GEMV_NO_FAST,
- * FLUTE_GEMM_ROWS, FLUTE_GEMM_NO_PERM, FLUTE_GEMM_KSPLIT, FLUTE_GEMM_NO_DIRECT,
- * FLUTE_FHT_STEPS) from the environment once per process; this re-reads them.
+ * FLUTE_GEMV4_WALK, FLUTE_GEMM_ROWS, FLUTE_GEMM_NO_PERM, FLUTE_GEMM_KSPLIT,
+ * FLUTE_GEMM_NO_DIRECT, FLUTE_FHT_STEPS) from the environment once per process; this
+ * re-reads them.
  */
 void flute_reload_tuning(void);
 

@@ -312,7 +312,19 @@ flute_status launch_fast4(Plan &plan, hipStream_t stream) {
                                             (int)kLdsPerCU));
         attr_done = true;
     }
-    dim3 grid(plan.grid_x, plan.p.split);
+    // A grid of several rounds of workgroups: as many workgroups as are resident at once walk
+    // over the row slices instead, which stages the activations once per workgroup and lets a
+    // slice's first loads travel under the previous slice's last products.
+    int gx = plan.grid_x;
+    plan.p.slices = 0;
+    const int per_cu = tuning().gemv4_walk >= 0 ? tuning().gemv4_walk : (NW == 4 ? 3 : 2);
+    const int resident = per_cu * kNumCU;
+    if (per_cu > 0 && plan.p.split == 1 && (plan.p.nsegs == 1 || plan.p.silu_mul) &&
+        plan.lds_bytes * per_cu <= (size_t)kLdsPerCU && gx > resident) {
+        plan.p.slices = gx;
+        gx = resident;
+    }
+    dim3 grid(gx, plan.p.split);
     hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, PF, BF16>), grid, dim3(NW * 64), plan.lds_bytes,
                        stream, plan.p);
     FLUTE_HIP_CHECK(hipGetLastError());

@@ -184,9 +184,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const int kg = L >> 4, rb = (L >> 2) & 3, kt = L & 3;
     const int gsub = rb >> SH;                      // tile of the load this lane reads
     const int cgl = rb & ((1 << SH) - 1);           // chunk group inside the row slice
-    const int sl = (int)blockIdx.x - kp->seg[si0].col0;
-    const int t = sl / SPT;
-    const int cg0 = (sl % SPT) * (RW >> 3);
+    // The row slice of this workgroup; with p.slices set it walks on through the slices
+    // blockIdx.x + i * gridDim.x, keeping the staged activations.
+    int sl = (int)blockIdx.x - kp->seg[si0].col0;
+    const bool walk = p.slices > 0;                 // uniform; unsplit launches of one column space
     const int s = blockIdx.y;
     const int g_lo = s * p.gs_tiles;
     const int units = p.gs_tiles / GPI;
@@ -199,7 +200,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 
     // lane-constant pieces of the addresses
     const uint32_t unit_bytes = GPI * 4096u;
-    const uint32_t lane0 = (uint32_t)gsub * 4096u + (uint32_t)(cg0 + cgl) * 256u +
+    const uint32_t lane0 = (uint32_t)gsub * 4096u + (uint32_t)cgl * 256u +
                            (uint32_t)kg * 64u + (uint32_t)kt * 16u + (uint32_t)w * unit_bytes;
     constexpr uint32_t step = NW * GPI * 4096u;
     // Lookup addresses are formed as absolute LDS addresses, so the (zero) base of
@@ -220,11 +221,12 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // stream for a plain weight, two streams for a dual-stream weight, two outputs
     // for the gate/up pair.  Every pass covers the same K range with the same lane
     // geometry; only the index blob and the LUT row change.
-    auto pass_ptrs = [&](int so_, int si_, const uint8_t *&qr, const uint16_t *&lutp) {
+    auto pass_ptrs = [&](int sl_, int so_, int si_, const uint8_t *&qr, const uint16_t *&lutp) {
         const int sg = so_ == 1 ? 1 : si0;
         const GemvStream st = kp->seg[sg].st[si_];
+        const int t = sl_ / SPT, cg0 = (sl_ % SPT) * (RW >> 3);
         const int grp = min((t * 128) >> __builtin_ctz(kp->seg[sg].gs), kp->seg[sg].lut_rows - 1);
-        qr = st.q + ((size_t)t * G + g_lo) * 4096u;
+        qr = st.q + ((size_t)t * G + g_lo) * 4096u + (uint32_t)cg0 * 256u;
         lutp = st.lut + ((size_t)grp << 4);
     };
     // Index loads are addressed as (uniform base + unit offset) in scalar registers
@@ -274,7 +276,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     int so = 0, si = 0;
     const uint8_t *qrow;
     const uint16_t *lut;
-    pass_ptrs(0, 0, qrow, lut);
+    pass_ptrs(sl, 0, 0, qrow, lut);
     uint32_t lrow[8];
     load_lut_row(lut, lrow);
     const uint16_t *staged_x = kp->seg[si0].xsrc ? kp->seg[si0].xsrc : p.x;
@@ -415,6 +417,46 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const int xoff = (kg * GPI + gsub) * 4 + kt;    // operand order: 8-byte word of this lane
     const int xnat = gsub * 32 + kt * 8 + kg;       // natural order: first dword of this lane
 
+    // ---- one thread per owned row: fold the wavefronts and the tiles of a load, then the
+    //      residual, the bias, the gate and the store -----------------------------------
+    const int cgl_o = tid >> 3, a_o = tid & 7;
+    auto row_n = [&](int sl_) -> int {
+        return (sl_ / SPT) * 128 + row_of((sl_ % SPT) * (RW >> 3) + cgl_o, a_o);
+    };
+    auto fold_rows = [&](float (&yv)[2]) {
+        yv[0] = yv[1] = 0.0f;
+#pragma unroll
+        for (int so = 0; so < 2; ++so) {
+            if (so >= nout) break;
+            float y = 0.0f;
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww)
+#pragma unroll
+                for (int gb = 0; gb < GPI; ++gb)
+                    y += red[(so * NW + ww) * 32 + ((gb << SH) | cgl_o) * 8 + a_o];
+            yv[so] = y;
+        }
+    };
+    auto finish_rows = [&](int sl_, float (&yv)[2]) {
+        const int n = row_n(sl_);
+#pragma unroll
+        for (int so = 0; so < 2; ++so) {
+            if (so >= nout) break;
+            const GemvSeg og = kp->seg[so == 1 ? 1 : si0];
+            float y = yv[so];
+            if (og.R > 0) {
+                const uint16_t *ra = og.resA + (size_t)n * og.R;
+                for (int r = 0; r < og.R; ++r)
+                    y = fmaf(og.xb[r], p.act_bf16 ? bf2f(ra[r]) : h2f(ra[r]), y);
+            }
+            if (og.bias) y += p.act_bf16 ? bf2f(og.bias[n]) : h2f(og.bias[n]);
+            yv[so] = y;
+        }
+        float y = yv[0];
+        if (p.silu_mul) y = (yv[0] / (1.0f + expf(-yv[0]))) * yv[1];
+        kp->seg[si0].out[n] = round_act(y, p.act_bf16);
+    };
+
     for (bool first = true;; first = false) {
         const int sg = so == 1 ? 1 : si0;
         if (!first) {
@@ -427,16 +469,23 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         // ---- the pass after this one: its LUT row is fetched now and its first index
         //      loads replace this pass's last ones as they are consumed, so the memory
         //      stream does not stop between passes. -----------------------------------
-        int nso = so, nsi = si + 1;
+        int nso = so, nsi = si + 1, nsl = sl;
         if (nsi == kp->seg[sg].nstreams) {
             nsi = 0;
             nso = so + 1;
+        }
+        const bool out_ends = nso != so;
+        bool slice_ends = false;
+        if (nso == nout && walk && sl + (int)gridDim.x < p.slices) {
+            nsl = sl + (int)gridDim.x;              // on to the first pass of the next slice
+            nso = 0;
+            slice_ends = true;
         }
         const bool has_next = nso < nout;
         const uint8_t *qnext = qrow;
         const uint16_t *lutn = lut;
         if (has_next) {
-            pass_ptrs(nso, nsi, qnext, lutn);
+            pass_ptrs(nsl, nso, nsi, qnext, lutn);
             load_lut_row(lutn, lrow);
         }
         __syncthreads();
@@ -507,7 +556,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         // ---- end of an output: D[i][j] with i = (rb, kt) in (lane >> 4, register) and
         //      j = (rb', kt') in lane & 15.  The lanes with rb' == rb keep register kt';
         //      a quad sum folds kt'; the activation scaling is undone here (exact). -----
-        if (nso != so) {
+        if (out_ends) {
             const bool keep = rb == kg;             // here L >> 4 is the matrix row block
 #pragma unroll
             for (int a = 0; a < 8; ++a) {
@@ -521,6 +570,16 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         }
         if (!has_next) break;
         __syncthreads();                            // the table region is rewritten next
+        if (slice_ends) {
+            // The partial sums of the finished slice are complete behind the barrier above and
+            // are next written behind the one that publishes the coming table.
+            if (tid < RW) {
+                float yv[2];
+                fold_rows(yv);
+                finish_rows(sl, yv);
+            }
+            sl = nsl;
+        }
         so = nso;
         si = nsi;
         qrow = qnext;
@@ -528,25 +587,11 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     }
     __syncthreads();
 
-    // ---- one thread per owned row: fold the wavefronts and the tiles of a load ------
     if (tid >= RW && p.split == 1) return;
     const bool owner = tid < RW;
-    const int cgl_o = tid >> 3, a_o = tid & 7;
-    const int n = t * 128 + row_of(cg0 + cgl_o, a_o);
+    const int n = row_n(sl);
     float yv[2] = {0.0f, 0.0f};
-    if (owner) {
-#pragma unroll
-        for (int so = 0; so < 2; ++so) {
-            if (so >= nout) break;
-            float y = 0.0f;
-#pragma unroll
-            for (int ww = 0; ww < NW; ++ww)
-#pragma unroll
-                for (int gb = 0; gb < GPI; ++gb)
-                    y += red[(so * NW + ww) * 32 + ((gb << SH) | cgl_o) * 8 + a_o];
-            yv[so] = y;
-        }
-    }
+    if (owner) fold_rows(yv);
 
     if (p.split > 1) {
         int *flag = (int *)(red + 2 * NW * 32);
@@ -590,24 +635,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                                __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    if (owner) {
-#pragma unroll
-        for (int so = 0; so < 2; ++so) {
-            if (so >= nout) break;
-            const GemvSeg og = kp->seg[so == 1 ? 1 : si0];
-            float y = yv[so];
-            if (og.R > 0) {
-                const uint16_t *ra = og.resA + (size_t)n * og.R;
-                for (int r = 0; r < og.R; ++r)
-                    y = fmaf(og.xb[r], p.act_bf16 ? bf2f(ra[r]) : h2f(ra[r]), y);
-            }
-            if (og.bias) y += p.act_bf16 ? bf2f(og.bias[n]) : h2f(og.bias[n]);
-            yv[so] = y;
-        }
-        float y = yv[0];
-        if (p.silu_mul) y = (yv[0] / (1.0f + expf(-yv[0]))) * yv[1];
-        kp->seg[si0].out[n] = round_act(y, p.act_bf16);
-    }
+    if (owner) finish_rows(sl, yv);
 }
 
 }  // namespace flute

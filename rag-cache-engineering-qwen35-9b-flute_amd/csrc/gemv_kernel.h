@@ -84,6 +84,7 @@ struct GemvParams {
     int fht_block;          // > 0: equal rotation blocks of this many columns
     int lds_x;              // LDS byte offsets
     int lds_red;
+    int slices;             // > 0: a workgroup walks the row slices blockIdx.x, + gridDim.x, ... below this
 };
 
 // Reads one dword of every 64-byte line of the kernel-argument block with

@@ -334,6 +334,51 @@ def test_long_k_narrow_output_takes_the_library_s_split():
     assert rel_l2(y.cpu(), _exact(w, x).half()) <= TOL
 
 
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,bits2,rank,bias", [(12288, 0, 0, False), (4224, 0, 0, False),
+                                              (4224, 4, 8, True)])
+def test_resident_grid_walking_the_row_slices(tuning_env, N, bits2, rank, bias, act):
+    """Launches of more workgroups than the device holds at once run as a resident grid whose
+    workgroups walk over the row slices (the very wide outputs of upstream's lm_head class,
+    src/kernel_gemv.cu:92-253, on one staged activation vector).  FLUTE_GEMV4_WALK sets the
+    resident workgroups per CU: 1 makes these sizes walk (three slices each; 528 slices over 256
+    workgroups, so sixteen workgroups take a third one), 0 switches walking off.  Same sums in
+    the same order: bit-identical outputs, and within tolerance of the oracle."""
+    K = 2048
+    w = make_weight(N, K, 4, 128, seed=61, bits2=bits2, rank=rank, bias=bias, act_dtype=act, device=DEV)
+    x = make_x(1, K, seed=62, dtype=act)
+    tuning_env("FLUTE_GEMV4_WALK", "0")
+    plain = _run(w, x)
+    tuning_env("FLUTE_GEMV4_WALK", "1")
+    walked = _run(w, x)
+    assert torch.equal(plain, walked)
+    # bfloat16 outputs: the rounding of the output alone is 1.6e-3
+    assert rel_l2(walked.cpu(), _exact(w, x).to(act)) <= (TOL if act == torch.float16 else 4e-3)
+
+
+def test_resident_grid_walking_the_merged_gate_up(tuning_env):
+    """The merged gate/up launch (two index streams per slice, SiLU(gate) * up at the end of a
+    slice) on a walking grid: bit-identical to the unwalked launch."""
+    N, K = 4224, 2048
+    g = make_weight(N, K, 4, 128, seed=63, device=DEV)
+    u = make_weight(N, K, 4, 128, seed=64, device=DEV)
+    x = make_x(1, K, seed=65)
+    table = torch.tensor([[g["blob_d"].data_ptr(), g["lut_d"].data_ptr(), 0, 0, 0, 0, 0, 0, N, 0, 4, 0,
+                           128, 0, 0],
+                          [u["blob_d"].data_ptr(), u["lut_d"].data_ptr(), 0, 0, 0, 0, 0, 0, N, 0, 4, 0,
+                           128, 0, 0]], dtype=torch.int64)
+    outs = []
+    for walk in ("0", "1"):
+        tuning_env("FLUTE_GEMV4_WALK", walk)
+        out = torch.zeros(1, N, dtype=torch.float16, device=DEV)
+        fx.qgemm_gemv_mlp(x.to(DEV), table, out)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    yg = O.linear_exact(x, g["blob"].numpy(), g["lut"], N, K, 128, 4)
+    yu = O.linear_exact(x, u["blob"].numpy(), u["lut"], N, K, 128, 4)
+    assert rel_l2(outs[1].cpu(), O.silu_mul_exact(yg, yu).half()) <= TOL
+
+
 def test_two_streams_share_the_workspace_in_order():
     """The split-K workspace is one per device (upstream: one stream only,
     src/gemv_host.h:31-38).  Launches that alternate between two streams, with nothing but the
