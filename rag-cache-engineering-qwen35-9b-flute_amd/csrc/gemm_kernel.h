@@ -517,6 +517,12 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 load_tile();                              // second tile (or a harmless reload)
             }
             while (left > 0) {
+                // The two wavefronts of a SIMD (wavefront w and w + 4) take turns at the higher
+                // priority, tile by tile: each then runs its products of a tile in one stretch
+                // while the other waits for its loads, instead of both interleaving and both
+                // waiting (M = 256, 4096 -> 12288: 42.0 -> 39.3 us).
+                if ((left + (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(0);
                 stage_read();                             // this tile's chunk
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (DIRECT) {
@@ -544,6 +550,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 __builtin_amdgcn_sched_barrier(0);
                 --left;
             }
+            __builtin_amdgcn_s_setprio(0);
         } else if constexpr (B1 > 0) {
             uint32_t lb[4];
             table_bases(lb, 0, B1);
