@@ -303,32 +303,39 @@ flute_status launch_typed(Plan &plan, hipStream_t stream) {
     return FLUTE_OK;
 }
 
-template <int LPGL, int NW, int PF, bool BF16>
-flute_status launch_fast4(Plan &plan, hipStream_t stream) {
+template <int LPGL, int NW, int PF, bool BF16, bool WALK>
+flute_status launch_fast4_grid(const Plan &plan, int gx, hipStream_t stream) {
     static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv4_kernel<LPGL, NW, PF, BF16>,
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv4_kernel<LPGL, NW, PF, BF16, WALK>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
                                             (int)kLdsPerCU));
         attr_done = true;
     }
+    dim3 grid(gx, plan.p.split);
+    hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, PF, BF16, WALK>), grid, dim3(NW * 64), plan.lds_bytes,
+                       stream, plan.p);
+    FLUTE_HIP_CHECK(hipGetLastError());
+    return FLUTE_OK;
+}
+
+template <int LPGL, int NW, int PF, bool BF16>
+flute_status launch_fast4(Plan &plan, hipStream_t stream) {
     // A grid of several rounds of workgroups: as many workgroups as are resident at once walk
     // over the row slices instead, which stages the activations once per workgroup and lets a
     // slice's first loads travel under the previous slice's last products.
     int gx = plan.grid_x;
     plan.p.slices = 0;
-    const int per_cu = tuning().gemv4_walk >= 0 ? tuning().gemv4_walk : (NW == 4 ? 3 : 2);
-    const int resident = per_cu * kNumCU;
-    if (per_cu > 0 && plan.p.split == 1 && (plan.p.nsegs == 1 || plan.p.silu_mul) &&
-        plan.lds_bytes * per_cu <= (size_t)kLdsPerCU && gx > resident) {
-        plan.p.slices = gx;
-        gx = resident;
+    if constexpr (NW == 4) {                     // (eight-wavefront workgroups serve short grids only)
+        const int per_cu = tuning().gemv4_walk >= 0 ? tuning().gemv4_walk : 3;
+        const int resident = per_cu * kNumCU;
+        if (per_cu > 0 && plan.p.split == 1 && (plan.p.nsegs == 1 || plan.p.silu_mul) &&
+            plan.lds_bytes * per_cu <= (size_t)kLdsPerCU && gx > resident) {
+            plan.p.slices = gx;
+            return launch_fast4_grid<LPGL, NW, PF, BF16, true>(plan, resident, stream);
+        }
     }
-    dim3 grid(gx, plan.p.split);
-    hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, PF, BF16>), grid, dim3(NW * 64), plan.lds_bytes,
-                       stream, plan.p);
-    FLUTE_HIP_CHECK(hipGetLastError());
-    return FLUTE_OK;
+    return launch_fast4_grid<LPGL, NW, PF, BF16, false>(plan, gx, stream);
 }
 
 // Loads a lane keeps in flight in the lean kernel: 4 when that divides the loads of a

@@ -149,7 +149,9 @@ __device__ __forceinline__ void rotate_piece(uint4 &v, const float (&sg)[8], con
 //        and even (two loads feed one matrix product).
 // The table stride is 128 bytes (32 replicas of a 4-byte entry, 32 KB): three
 // four-wavefront workgroups fit a CU.
-template <int LPGL, int NW, int PF, bool BF16>
+// WALK: the instantiation for resident grids that walk over the row slices (p.slices > 0);
+// launches of one workgroup per slice use the one without that control path.
+template <int LPGL, int NW, int PF, bool BF16, bool WALK = false>
 __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int ES = 7;
@@ -187,7 +189,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // The row slice of this workgroup; with p.slices set it walks on through the slices
     // blockIdx.x + i * gridDim.x, keeping the staged activations.
     int sl = (int)blockIdx.x - kp->seg[si0].col0;
-    const bool walk = p.slices > 0;                 // uniform; unsplit launches of one column space
+    constexpr bool walk = WALK;                     // unsplit launches of one column space
     const int s = blockIdx.y;
     const int g_lo = s * p.gs_tiles;
     const int units = p.gs_tiles / GPI;
