@@ -518,9 +518,8 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             }
             while (left > 0) {
                 // The two wavefronts of a SIMD (wavefront w and w + 4) take turns at the higher
-                // priority, tile by tile: each then runs its products of a tile in one stretch
-                // while the other waits for its loads, instead of both interleaving and both
-                // waiting (M = 256, 4096 -> 12288: 42.0 -> 39.3 us).
+                // priority, tile by tile, so that neither falls a tile behind the other
+                // (measured with the builds interleaved: about 1 % at M = 256 and M = 1024).
                 if ((left + (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1);
                 else __builtin_amdgcn_s_setprio(0);
                 stage_read();                             // this tile's chunk
