@@ -356,6 +356,23 @@ def test_resident_grid_walking_the_row_slices(tuning_env, N, bits2, rank, bias, 
     assert rel_l2(walked.cpu(), _exact(w, x).to(act)) <= (TOL if act == torch.float16 else 4e-3)
 
 
+@pytest.mark.parametrize("block", [128, 1024, 0])
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+def test_resident_grid_walking_with_a_rotated_input(tuning_env, block, act):
+    """The input rotation runs once, in the prologue of a walking workgroup (in the consuming
+    wavefront's registers for block 128, through the LDS buffer that the first table then
+    overwrites for block 1024 and for the whole-row transform): same bits as the unwalked launch."""
+    N, K = 4224, 2048
+    w = make_weight(N, K, 4, 128, seed=66, act_dtype=act, device=DEV)
+    x = make_x(1, K, seed=67, dtype=act)
+    signs = O.rotation_signs(K, block)              # the second argument is the seed
+    extra = {"rot_block": block} if block else {}
+    tuning_env("FLUTE_GEMV4_WALK", "0")
+    plain = _run(w, x, signs=signs, **extra)
+    tuning_env("FLUTE_GEMV4_WALK", "1")
+    assert torch.equal(plain, _run(w, x, signs=signs, **extra))
+
+
 def test_resident_grid_walking_the_merged_gate_up(tuning_env):
     """The merged gate/up launch (two index streams per slice, SiLU(gate) * up at the end of a
     slice) on a walking grid: bit-identical to the unwalked launch."""
