@@ -34,6 +34,14 @@
 // The LUT row (32 bytes) comes through the scalar cache, so it does not queue
 // behind the index loads of the other workgroups of the CU in the vector memory
 // pipe; index loads are non-temporal (read once).
+//
+// Walking grids (template argument WALK).  A launch with more row slices than workgroups
+// fit the device at once (very wide outputs) is started as one resident workgroup per slot;
+// workgroup b takes the slices b, b + gridDim.x, ...  It stages the activations once; the
+// change of slice is handled like the change of stream inside a slice: the next slice's
+// LUT row and first index loads are requested under the last products of the current one,
+// the owners of the finished rows fold and store them while the other wavefronts write the
+// next table.  The sums of a row are formed in the same order as in a one-slice launch.
 #pragma once
 
 #include "gemv_kernel.h"
