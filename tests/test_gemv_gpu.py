@@ -373,6 +373,26 @@ def test_resident_grid_walking_with_a_rotated_input(tuning_env, block, act):
     assert torch.equal(plain, _run(w, x, signs=signs, **extra))
 
 
+def test_very_wide_output_walks_by_the_library_s_own_choice(tuning_env):
+    """40960 rows are 1280 slices of 32 rows, more than the 768 workgroups the device holds: the
+    library walks without being told to.  Bit-identical to the launch of one workgroup per
+    slice, within tolerance of the oracle on every row, and a one-hot input returns the
+    dequantised column bit for bit (first, middle and last tile)."""
+    N, K = 40960, 1024
+    w = make_weight(N, K, 4, 128, seed=71, device=DEV)
+    x = make_x(1, K, seed=72)
+    walked = _run(w, x)
+    tuning_env("FLUTE_GEMV4_WALK", "0")
+    assert torch.equal(walked, _run(w, x))
+    tuning_env("FLUTE_GEMV4_WALK", None)
+    assert rel_l2(walked.cpu(), _exact(w, x).half()) <= TOL
+    Wd = O.dequant(w["blob"].numpy(), w["lut"], N, K, 128, 4)
+    for k in (0, 517, K - 1):
+        e = torch.zeros(1, K, dtype=torch.float16)
+        e[0, k] = 1.0
+        assert torch.equal(_run(w, e).cpu().view(-1), Wd[:, k].half())
+
+
 def test_resident_grid_walking_the_merged_gate_up(tuning_env):
     """The merged gate/up launch (two index streams per slice, SiLU(gate) * up at the end of a
     slice) on a walking grid: bit-identical to the unwalked launch."""
