@@ -327,7 +327,8 @@ flute_status launch_fast4(Plan &plan, hipStream_t stream) {
     int gx = plan.grid_x;
     plan.p.slices = 0;
     if constexpr (NW == 4) {                     // (eight-wavefront workgroups serve short grids only)
-        const int per_cu = tuning().gemv4_walk >= 0 ? tuning().gemv4_walk : 3;
+        // three workgroups per CU is what the kernel's registers allow (3 wavefronts per SIMD)
+        const int per_cu = tuning().gemv4_walk >= 0 ? (tuning().gemv4_walk < 3 ? tuning().gemv4_walk : 3) : 3;
         const int resident = per_cu * kNumCU;
         if (per_cu > 0 && plan.p.split == 1 && (plan.p.nsegs == 1 || plan.p.silu_mul) &&
             plan.lds_bytes * per_cu <= (size_t)kLdsPerCU && gx > resident) {
