@@ -64,6 +64,14 @@ __device__ __forceinline__ gv_f4_t gv_mfma(gv_u4_t a, gv_u4_t b, gv_f4_t c) {
     }
 }
 
+// The value that lane (CTRL & 3) of this lane's quad holds (CTRL = that lane number in all four
+// two-bit fields of a quad_perm control).
+template <int CTRL>
+__device__ __forceinline__ float quad_lane(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
 // Sixteen index bytes, read once: non-temporal, so they do not displace the
 // activations and LUT rows that every workgroup shares from the caches.
 __device__ __forceinline__ uint4 load_idx16(const uint8_t *p) {
@@ -570,10 +578,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             const bool keep = rb == kg;             // here L >> 4 is the matrix row block
 #pragma unroll
             for (int a = 0; a < 8; ++a) {
-                float v = kt == 0 ? acc[a][0] : kt == 1 ? acc[a][1] : kt == 2 ? acc[a][2] : acc[a][3];
-                v = keep ? v : 0.0f;
-                v = dpp_add<0xB1>(v);               // quad_perm [1,0,3,2]
-                v = dpp_add<0x4E>(v);               // quad_perm [2,3,0,1]
+                // lane kt' of a quad holds the wanted term in register kt': each register is
+                // read from its own lane of the quad, summed as (0 + 1) + (2 + 3)
+                const float v = (quad_lane<0x00>(acc[a][0]) + quad_lane<0x55>(acc[a][1])) +
+                                (quad_lane<0xAA>(acc[a][2]) + quad_lane<0xFF>(acc[a][3]));
                 if (keep && kt == 0) red[(so * NW + w) * 32 + rb * 8 + a] = ldexpf(v, xshift);
                 acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
             }
