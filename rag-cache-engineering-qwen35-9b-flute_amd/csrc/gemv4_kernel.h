@@ -37,11 +37,15 @@
 //
 // Walking grids (template argument WALK).  A launch with more row slices than workgroups
 // fit the device at once (very wide outputs) is started as one resident workgroup per slot;
-// workgroup b takes the slices b, b + gridDim.x, ...  It stages the activations once; the
-// change of slice is handled like the change of stream inside a slice: the next slice's
-// LUT row and first index loads are requested under the last products of the current one,
-// the owners of the finished rows fold and store them while the other wavefronts write the
-// next table.  The sums of a row are formed in the same order as in a one-slice launch.
+// with four slices or more each a workgroup takes a contiguous run of them (consecutive
+// slices mostly share a 128-row tile, hence the LUT row, and the table is then kept instead
+// of rebuilt; the partial row sums alternate between two LDS areas so that the barrier
+// which would publish the table can go too), with fewer it takes b, b + gridDim.x, ...
+// It stages the activations once; the change of slice is handled like the change of stream
+// inside a slice: the next slice's LUT row and first index loads are requested under the
+// last products of the current one, the owners of the finished rows fold and store them
+// while the other wavefronts go on.  The sums of a row are formed in the same order as in
+// a one-slice launch.
 #pragma once
 
 #include "gemv_kernel.h"
@@ -185,6 +189,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     constexpr int CPT = CHUNKS / SHARES;            // pieces written per thread
     static_assert(NT >= 256, "one thread per table entry at least");
     static_assert(PF % 2 == 0 && PF >= PF0, "loads are consumed in pairs");
+    static_assert(!WALK || NW == 4, "the alternating sum areas of a walking grid are sized for four wavefronts");
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     warm_kernargs<(int)sizeof(GemvParams)>(kp);
@@ -202,10 +207,26 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const int kg = L >> 4, rb = (L >> 2) & 3, kt = L & 3;
     const int gsub = rb >> SH;                      // tile of the load this lane reads
     const int cgl = rb & ((1 << SH) - 1);           // chunk group inside the row slice
-    // The row slice of this workgroup; with p.slices set it walks on through the slices
-    // blockIdx.x + i * gridDim.x, keeping the staged activations.
-    int sl = (int)blockIdx.x - kp->seg[si0].col0;
+    // The row slice of this workgroup.  A walking workgroup keeps the staged activations and
+    // takes, from four slices per workgroup on, a contiguous run of the p.slices slices (the
+    // first p.slices % gridDim.x workgroups one more than the others): consecutive slices
+    // mostly lie in one 128-row tile and then share their LUT row, i.e. their table.  With
+    // fewer slices each it takes blockIdx.x, + gridDim.x, ...: the neighbours then read the
+    // four slices of a tile at the same time, which the memory system likes better.
     constexpr bool walk = WALK;                     // unsplit launches of one column space
+    int sl = (int)blockIdx.x - kp->seg[si0].col0;
+    int sl_end = sl + 1, sl_step = 1;
+    if constexpr (walk) {
+        const int per = p.slices / (int)gridDim.x, extra = p.slices % (int)gridDim.x;
+        const int b = (int)blockIdx.x;
+        if (per >= 4) {
+            sl = b * per + min(b, extra);
+            sl_end = sl + per + (b < extra ? 1 : 0);
+        } else {
+            sl_end = p.slices;
+            sl_step = (int)gridDim.x;
+        }
+    }
     const int s = blockIdx.y;
     const int g_lo = s * p.gs_tiles;
     const int units = p.gs_tiles / GPI;
@@ -441,7 +462,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     auto row_n = [&](int sl_) -> int {
         return (sl_ / SPT) * 128 + row_of((sl_ % SPT) * (RW >> 3) + cgl_o, a_o);
     };
-    auto fold_rows = [&](float (&yv)[2]) {
+    auto fold_rows = [&](float (&yv)[2], int par_) {
         yv[0] = yv[1] = 0.0f;
 #pragma unroll
         for (int so = 0; so < 2; ++so) {
@@ -451,7 +472,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             for (int ww = 0; ww < NW; ++ww)
 #pragma unroll
                 for (int gb = 0; gb < GPI; ++gb)
-                    y += red[(so * NW + ww) * 32 + ((gb << SH) | cgl_o) * 8 + a_o];
+                    y += red[par_ * (2 * NW * 32) + (so * NW + ww) * 32 + ((gb << SH) | cgl_o) * 8 + a_o];
             yv[so] = y;
         }
     };
@@ -475,9 +496,11 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         kp->seg[si0].out[n] = round_act(y, p.act_bf16);
     };
 
+    bool same_table = false;                        // walking: the next slice reuses the table
+    int par = 0;                                    // walking: the partial sums alternate between two areas
     for (bool first = true;; first = false) {
         const int sg = so == 1 ? 1 : si0;
-        if (!first) {
+        if (!first && !same_table) {
             // every output of the launch reads the same staged activations (the host
             // sends launches whose outputs differ in input or rotation to the general
             // kernel), so only the table changes between passes
@@ -494,19 +517,23 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         }
         const bool out_ends = nso != so;
         bool slice_ends = false;
-        if (nso == nout && walk && sl + (int)gridDim.x < p.slices) {
-            nsl = sl + (int)gridDim.x;              // on to the first pass of the next slice
+        if (nso == nout && walk && sl + sl_step < sl_end) {
+            nsl = sl + sl_step;                     // on to the first pass of the next slice
             nso = 0;
             slice_ends = true;
         }
         const bool has_next = nso < nout;
         const uint8_t *qnext = qrow;
         const uint16_t *lutn = lut;
+        bool next_same = false;
         if (has_next) {
             pass_ptrs(nsl, nso, nsi, qnext, lutn);
-            load_lut_row(lutn, lrow);
+            // one output of one stream per slice and the same LUT row: the table stands
+            next_same = walk && slice_ends && nout == 1 && kp->seg[sg].nstreams == 1 && lutn == lut;
+            if (!next_same) load_lut_row(lutn, lrow);
         }
-        __syncthreads();
+        // publishes the table; with the table kept, the alternating sum areas make it unnecessary
+        if (!same_table) __syncthreads();
 
         // ---- K loop -----------------------------------------------------------------
         // One step = two 16-byte loads of this lane = 32 lookups and 8 matrix products.
@@ -582,22 +609,25 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 // read from its own lane of the quad, summed as (0 + 1) + (2 + 3)
                 const float v = (quad_lane<0x00>(acc[a][0]) + quad_lane<0x55>(acc[a][1])) +
                                 (quad_lane<0xAA>(acc[a][2]) + quad_lane<0xFF>(acc[a][3]));
-                if (keep && kt == 0) red[(so * NW + w) * 32 + rb * 8 + a] = ldexpf(v, xshift);
+                if (keep && kt == 0)
+                    red[par * (2 * NW * 32) + (so * NW + w) * 32 + rb * 8 + a] = ldexpf(v, xshift);
                 acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
         if (!has_next) break;
         __syncthreads();                            // the table region is rewritten next
         if (slice_ends) {
-            // The partial sums of the finished slice are complete behind the barrier above and
-            // are next written behind the one that publishes the coming table.
+            // The partial sums of the finished slice are complete behind the barrier above; the
+            // next slice writes the other area, and this one again only two barriers later.
             if (tid < RW) {
                 float yv[2];
-                fold_rows(yv);
+                fold_rows(yv, par);
                 finish_rows(sl, yv);
             }
             sl = nsl;
+            par ^= 1;
         }
+        same_table = next_same;
         so = nso;
         si = nsi;
         qrow = qnext;
@@ -609,7 +639,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const bool owner = tid < RW;
     const int n = row_n(sl);
     float yv[2] = {0.0f, 0.0f};
-    if (owner) fold_rows(yv);
+    if (owner) fold_rows(yv, par);
 
     if (p.split > 1) {
         int *flag = (int *)(red + 2 * NW * 32);

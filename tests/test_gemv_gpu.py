@@ -336,15 +336,18 @@ def test_long_k_narrow_output_takes_the_library_s_split():
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N,bits2,rank,bias", [(12288, 0, 0, False), (4224, 0, 0, False),
-                                              (4224, 4, 8, True)])
+                                              (4224, 4, 8, True), (33024, 0, 8, True),
+                                              (33024, 4, 0, False)])
 def test_resident_grid_walking_the_row_slices(tuning_env, N, bits2, rank, bias, act):
     """Launches of more workgroups than the device holds at once run as a resident grid whose
     workgroups walk over the row slices (the very wide outputs of upstream's lm_head class,
     src/kernel_gemv.cu:92-253, on one staged activation vector).  FLUTE_GEMV4_WALK sets the
     resident workgroups per CU: 1 makes these sizes walk (three slices each; 528 slices over 256
-    workgroups, so sixteen workgroups take a third one), 0 switches walking off.  Same sums in
-    the same order: bit-identical outputs, and within tolerance of the oracle."""
-    K = 2048
+    workgroups, so sixteen workgroups take a third one), 0 switches walking off.  33024 rows are
+    1032 slices of 32 rows: four or five in a row per workgroup, which keeps its table while the
+    LUT row stays the same (one stream) and rebuilds it per stream (two).  Same sums in the same
+    order: bit-identical outputs, and within tolerance of the oracle."""
+    K = 2048 if N < 30000 else 1024
     w = make_weight(N, K, 4, 128, seed=61, bits2=bits2, rank=rank, bias=bias, act_dtype=act, device=DEV)
     x = make_x(1, K, seed=62, dtype=act)
     tuning_env("FLUTE_GEMV4_WALK", "0")
