@@ -148,9 +148,15 @@ def _read_residual(meta: Dict, artifacts_dir: str, ctx: str, N: int, K: int):
     _check_sha(a_path, res.get("sha256_resA"), ctx)
     _check_sha(b_path, res.get("sha256_resB"), ctx)
     rank = int(res["rank"])
-    A = torch.from_numpy(np.fromfile(a_path, dtype=np.float16).copy()).view(N, rank)
-    B = torch.from_numpy(np.fromfile(b_path, dtype=np.float16).copy()).view(rank, K)
-    return A, B
+    factors = []
+    for path, rows, cols, which in ((a_path, N, rank, "resA"), (b_path, rank, K, "resB")):
+        flat = np.fromfile(path, dtype=np.float16)
+        if rank <= 0 or flat.size != rows * cols:
+            raise ValueError(f"{ctx}: {which} file {os.path.basename(path)} holds {flat.size} "
+                             f"float16 values, expected [{rows}, {cols}] for rank {rank} "
+                             f"(N={N}, K={K})")
+        factors.append(torch.from_numpy(flat.copy()).view(rows, cols))
+    return factors[0], factors[1]
 
 
 def _read_stream2(meta: Dict, artifacts_dir: str, ctx: str, N: int, K: int, bitwidth: int,
@@ -396,7 +402,7 @@ def replace_linear_with_palettized(model, metadata: Dict, artifacts_dir: str,
             setattr(holder, leaf, lm)
             holder, leaf = resolve_module(model, "model.embed_tokens.weight")
             setattr(holder, leaf, emb)
-            compensated += getattr(lm, "fold_order", None) == "rotate_then_awq"
+            compensated += lm._compensated()
             continue
         holder, leaf = resolve_module(model, name)
         old = getattr(holder, leaf)
@@ -409,8 +415,7 @@ def replace_linear_with_palettized(model, metadata: Dict, artifacts_dir: str,
                                          residual=residual, reference=reference,
                                          verify_sha=verify_sha, awq_scales=awq_scales)
             members = (new.q_proj, new.k_proj, new.v_proj) if isinstance(new, SplitQKV) else (new,)
-            compensated += sum(getattr(m, "fold_order", None) == "rotate_then_awq"
-                               for m in members)
+            compensated += sum(m._compensated() for m in members)
         setattr(holder, leaf, new)
     if compensated:
         print(f"  [ROT] rotate-then-AWQ fold order compensated on {compensated} tensor group(s)",

@@ -398,10 +398,13 @@ Tensor qgemm_gemv_mlp(const Tensor &A_in, const Tensor &seg_table, const Tensor 
     check_seg_inputs(who, A_in, seg_table, 2);
     TORCH_CHECK(C.scalar_type() == A_in.scalar_type() && C.is_contiguous(), who,
                 ": C must be a contiguous ", dtype_name(A_in), " output buffer");
-    const int64_t *v = seg_table.contiguous().data_ptr<int64_t>();
+    const Tensor table = seg_table.contiguous();   // alive while v is read
+    const int64_t *v = table.data_ptr<int64_t>();
     const int64_t N = v[8];
     TORCH_CHECK(v[kSegCols + 8] == N && C.numel() == N, who, ": gate/up/C must agree in N");
     TORCH_CHECK(A_in.is_cuda() && C.is_cuda(), who, ": A and C must be CUDA (HIP) tensors");
+    TORCH_CHECK(C.device() == A_in.device(), who, ": C must live on A's device ",
+                A_in.device().str());
     std::vector<flute_linear> descs;
     std::vector<void *> outs;
     seg_descs(who, A_in, seg_table, lut_code(lut_dtype), descs, outs);

@@ -363,6 +363,8 @@ def qgemm_gemv_mlp(A, seg_table, C, lut_dtype: Optional[torch.dtype] = None, spl
         _fail(f"{who}: gate/up/C must agree in N")
     if not (A.is_cuda and C.is_cuda):
         _fail(f"{who}: A and C must be CUDA (HIP) tensors")
+    if C.device != A.device:
+        _fail(f"{who}: C must live on A's device {A.device}")
     descs, _ = _seg_descs(who, A, seg_table, _ACT[lut_dtype or torch.float16])
     A = _aligned16(A)
     with _on_device_of(A):
@@ -439,6 +441,8 @@ def qgemm_debug_simple(A, indices, lut, bitwidth, group_size, q_layout: int = 0)
         _fail(f"{who}: bitwidth must be 1, 2, 3 or 4 (got {b})")
     if indices.dtype != torch.uint8 or not indices.is_contiguous() or not indices.is_cuda:
         _fail(f"{who}: indices must be a contiguous uint8 tensor on the GPU")
+    if not A.is_cuda or indices.device != A.device:
+        _fail(f"{who}: A and indices must live on the same GPU")
     if lut.dtype not in _ACT or lut.dim() != 2 or lut.shape[1] != (1 << b) or \
             not lut.is_contiguous() or lut.device != A.device:
         _fail(f"{who}: lut must be a contiguous [groups, 2^bitwidth] float16/bfloat16 tensor on "
@@ -506,6 +510,8 @@ def _fht(who, x, signs, awq, out, adjoint, block=0):
         _fail(f"{who}: x must be contiguous")
     if not (x.is_cuda and signs.is_cuda and (awq is None or awq.is_cuda)):
         _fail(f"{who}: all tensors must be CUDA (HIP) tensors")
+    if signs.device != x.device or (awq is not None and awq.device != x.device):
+        _fail(f"{who}: all tensors must live on x's device {x.device}")
     with _on_device_of(x):
         if out is None:
             out = torch.empty_like(x)

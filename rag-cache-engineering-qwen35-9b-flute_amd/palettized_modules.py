@@ -416,9 +416,9 @@ def _operand_ptrs(members) -> tuple:
     changes (a module moved to another device and back, a buffer replaced)."""
     out = []
     for m in members:
-        for t in (m.indices, m.lut, getattr(m, "indices2", None), getattr(m, "lut2", None),
-                  getattr(m, "resA", None), getattr(m, "resB", None), getattr(m, "bias", None)):
-            out.append(0 if t is None else t.data_ptr())
+        for name in ("indices", "lut", "indices2", "lut2", "resA", "resB", "bias"):
+            t = getattr(m, name, None)
+            out.append(t.data_ptr() if torch.is_tensor(t) else 0)
     return tuple(out)
 
 
@@ -468,9 +468,7 @@ class FusedPalettizedMLP(nn.Module):
         """Fusion verdict, persistent output and the CPU segment table, once per
         (device, dtype).  `reason` says why a pair is not fused."""
         g, u = self.gate_proj, self.up_proj
-        state = {"ok": False, "device": device, "dtype": dtype}
-        if isinstance(g, PalettizedLinear) and isinstance(u, PalettizedLinear):
-            state["ptrs"] = _operand_ptrs((g, u))
+        state = {"ok": False, "device": device, "dtype": dtype, "ptrs": _operand_ptrs((g, u))}
 
         def refuse(why):
             state["reason"] = why
@@ -569,9 +567,7 @@ class SplitQKV(nn.Module):
 
     def _build_state(self, device, dtype):
         members = (self.q_proj, self.k_proj, self.v_proj)
-        state = {"ok": False, "device": device, "dtype": dtype}
-        if all(isinstance(m, PalettizedLinear) for m in members):
-            state["ptrs"] = _operand_ptrs(members)
+        state = {"ok": False, "device": device, "dtype": dtype, "ptrs": _operand_ptrs(members)}
 
         def refuse(why):
             state["reason"] = why

@@ -107,6 +107,13 @@ def test_refusals(tmp_path):
     with pytest.raises(ValueError, match="expected"):
         artifacts.load_palettized_weight(dict(meta, dense_shape=[256, 64]), tmp, reference=True,
                                          verify_sha=False)
+    wr = make_weight(128, 64, bits=4, seed=8, rank=4)
+    mr = _write(tmp, "res", wr, residual=True)
+    artifacts.load_palettized_weight(mr, tmp, residual=True, reference=True)
+    short = dict(mr, residual=dict(mr["residual"], rank=8, sha256_resA=None, sha256_resB=None))
+    with pytest.raises(ValueError, match=r"resA file res.resA holds 512 float16 values, expected "
+                                         r"\[128, 8\]"):
+        artifacts.load_palettized_weight(short, tmp, residual=True, reference=True)
     os.remove(os.path.join(tmp, "r.lut_scalar.2"))
     with pytest.raises(ValueError, match="missing"):
         artifacts.load_palettized_weight(meta, tmp, reference=True)

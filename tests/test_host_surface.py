@@ -376,3 +376,11 @@ def test_merged_modules_refuse_operands_they_cannot_pass_by_address():
     before = pm._operand_ptrs((m,))
     m.indices = m.indices.clone()
     assert pm._operand_ptrs((m,)) != before
+    # members that are not palettized at all (a dense layer left in place) have no blobs: the
+    # tuple is still defined, and the verdict is a refusal that carries it
+    dense = torch.nn.Linear(128, 256)
+    assert pm._operand_ptrs((dense,))[:4] == (0, 0, 0, 0)
+    for wrapper in (pm.FusedPalettizedMLP(dense, member(wu), member(wg), silu),
+                    pm.SplitQKV(dense, member(wu), member(wg))):
+        state = wrapper._build_state(cpu, torch.float16)
+        assert state["reason"] == "non-PalettizedLinear member" and "ptrs" in state
