@@ -273,7 +273,10 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     region0 = (region0 + 255) & ~(size_t)255;
     p.lds_x = (int)region0;
     p.lds_red = p.lds_x + ((kc * 2 + 15) & ~15);
-    plan->lds_bytes = (size_t)p.lds_red + 2 * 8 * 32 * 4 + 16;
+    // row sums [2][8][32], the ticket flag (16 bytes), then one word per wavefront for the
+    // row maximum of a bfloat16 slice (not the row-sum area: a merged launch restages for its
+    // second output while the first output's sums are still waiting to be folded)
+    plan->lds_bytes = (size_t)p.lds_red + kGemvRedBytes + 16 + 8 * 4;
     FLUTE_REQUIRE(plan->lds_bytes <= (size_t)kLdsPerCU, FLUTE_ERR_UNSUPPORTED,
                   "%s: K=%d at split %d needs %zu B of LDS (limit %d)", who, K, split,
                   plan->lds_bytes, kLdsPerCU);

@@ -68,6 +68,8 @@ struct GemvSeg {            // one weight
     int ticket0;            // first ticket of this weight
 };
 
+constexpr int kGemvRedBytes = 2 * 8 * 32 * 4;   // partial row sums of two outputs, eight wavefronts
+
 struct GemvParams {
     GemvSeg seg[kGemvMaxSegs];
     const uint16_t *x;      // (K,) activations
@@ -83,7 +85,7 @@ struct GemvParams {
     int act_bf16;           // activations, residual, bias and outputs are bf16
     int fht_block;          // > 0: equal rotation blocks of this many columns
     int lds_x;              // LDS byte offsets
-    int lds_red;
+    int lds_red;            // row sums [2][8][32] fp32, ticket flag (16 B), 8 words for a row maximum
     int slices;             // > 0: a workgroup walks the row slices blockIdx.x, + gridDim.x, ... below this
 };
 
@@ -569,7 +571,8 @@ __device__ int stage_x(const GemvParams &p, const uint16_t *x, const float *sign
     auto finish = [&]() -> int {
         int shift = 0;
         if (convert)
-            shift = normalise_staged_row(xs, kc, (uint32_t *)(lds + p.lds_red), tid, nthreads);
+            shift = normalise_staged_row(xs, kc, (uint32_t *)(lds + p.lds_red + kGemvRedBytes + 16),
+                                         tid, nthreads);
         __syncthreads();
         return shift;
     };

@@ -65,6 +65,39 @@ def test_merged_gate_up_with_different_rotations():
     assert rel_l2(y, ref) <= TOL
 
 
+@pytest.mark.parametrize("rank", [0, 8])
+def test_merged_gate_up_different_rotations_bfloat16_rows_float16_lut(rank):
+    """bfloat16 activations in front of float16 LUTs are scaled per staged row, and a member with
+    its own signs makes the launch stage the row a second time while the first output's partial
+    row sums still wait in LDS: the scaling's scratch words must not be those sums.  Every gate
+    row is checked (the first rows of each slice were the ones at risk), with magnitudes beyond
+    float16's range so the scaling is exercised."""
+    N, K = 512, 4096
+    bf = torch.bfloat16
+    g = make_weight(N, K, seed=11, rank=rank, act_dtype=bf, device=DEV)
+    u = make_weight(N, K, seed=12, rank=rank, act_dtype=bf, device=DEV)
+    x = (make_x(1, K, seed=13).float() * 3.0e5).to(bf)
+    sg, su = O.rotation_signs(K, 1).to(DEV), O.rotation_signs(K, 2).to(DEV)
+    out = torch.zeros(1, N, dtype=bf, device=DEV)
+    table = torch.tensor([_row(g, signs=sg), _row(u, signs=su)], dtype=torch.int64)
+    y = fx.qgemm_gemv_mlp(x.to(DEV), table, out).cpu()
+    yg = _exact(g, O.fht_reference(x, sg.cpu()))
+    yu = _exact(u, O.fht_reference(x, su.cpu()))
+    ref = O.silu_mul_exact(yg, yu)
+    assert torch.isfinite(y).all()
+    assert rel_l2(y, ref.to(bf)) <= TOL           # same rounding point as the reference forward
+    # row by row: one bfloat16 rounding (2^-9) of a value whose factors are exact to ~1e-6
+    # (values far below bfloat16's normal range, where SiLU of a large negative sum underflows,
+    # are left to the norm above)
+    big = ref.double().abs() > 1e-30
+    err = (y.double() - ref.double()).abs()[big] / ref.double().abs()[big]
+    assert int(big.sum()) > N // 4 and float(err.max()) <= 2.0 ** -8
+    # each member alone through the single-weight entry gives the same sums
+    yg1 = fx.qgemm_gemv_stream(x.to(DEV), g["blob_d"], g["lut_d"], 4, 128, rot_signs=sg,
+                               **({"resA": g["resA_d"], "resB": g["resB_d"]} if rank else {})).cpu()
+    assert rel_l2(yg1, yg.to(bf)) <= TOL
+
+
 def test_grouped_launch():
     K = 2048
     ws = [make_weight(512, K, seed=1, device=DEV),
