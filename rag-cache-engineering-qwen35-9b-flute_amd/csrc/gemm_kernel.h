@@ -579,9 +579,10 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             };
             if constexpr (LEAN) {
                 // One round = one tile of this wavefront.  Vector memory instructions of a round,
-                // in issue order: the tile after next (4, into the LDS buffer just read out), the
-                // next tile's first-half operands (MB, one after each block of rows of this
-                // half), its second-half operands (MB).  Blocks of rows are outermost inside a
+                // in issue order: the next tile's first-half operand of the first block of rows, the
+                // tile after next (4, into the LDS buffer just read out), the other first-half
+                // operands (MB - 1, one after each block of rows of this half), the second-half
+                // operands (MB).  Blocks of rows are outermost inside a
                 // half: a block's activation operand is reloaded right after its eight
                 // products, a whole tile ahead of its use; the eight weight operands of a half
                 // stay in registers for all blocks, the last two blocks run side by side and
@@ -613,7 +614,10 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                             Q8[(q4 >> 1) * 4 + v], lb0, 0x03020000u | ((4u + d * 2 + (q4 & 1)) << 8));
                     return w;
                 };
-                auto half = [&](u4_t (&Aj)[MB], const u4_t *next) {
+                // `between` runs after the first block of rows (before the pair of blocks when
+                // there are only two): work that has to follow LDS reads issued in front of the
+                // half finds them complete there instead of waiting for them
+                auto half = [&](u4_t (&Aj)[MB], const u4_t *next, auto &&between) {
 #pragma unroll
                     for (int mb = 0; mb + 2 < MB; ++mb) {
 #pragma unroll
@@ -621,7 +625,9 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                         __builtin_amdgcn_sched_barrier(0);
                         lean_load16(Aj[mb], next, mb);
                         __builtin_amdgcn_sched_barrier(0);
+                        if (mb == 0) between();
                     }
+                    if constexpr (MB == 2) between();
 #pragma unroll
                     for (int o = 0; o < 8; ++o) {
                         acc[MB - 2][o] = mfma16<BF16>(W[o], Aj[MB - 2], acc[MB - 2][o]);
@@ -659,19 +665,23 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     // the second-half operands may still be in flight
                     wait_half(A0, std::integral_constant<int, MB>());
                     read_codes(1, cur);                   // this tile, second half
-                    asm volatile("s_waitcnt lgkmcnt(0)"
-                                 : "+v"(Q8[0]), "+v"(Q8[1]), "+v"(Q8[2]), "+v"(Q8[3]), "+v"(Q8[4]),
-                                   "+v"(Q8[5]), "+v"(Q8[6]), "+v"(Q8[7]) :: "memory");
-                    if (left > 2) lean_tq += qstep;
-                    lean_tile(cur != 0);                  // the tile after next, into the buffer just read
                     __builtin_amdgcn_sched_barrier(0);
-                    half(A0, apn);
+                    half(A0, apn, [&] {
+                        // the tile after next goes into the buffer just read out: not before
+                        // those reads have returned (one block of products later they have)
+                        asm volatile("s_waitcnt lgkmcnt(0)"
+                                     : "+v"(Q8[0]), "+v"(Q8[1]), "+v"(Q8[2]), "+v"(Q8[3]), "+v"(Q8[4]),
+                                       "+v"(Q8[5]), "+v"(Q8[6]), "+v"(Q8[7]) :: "memory");
+                        if (left > 2) lean_tq += qstep;
+                        lean_tile(cur != 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
                     // second-half operands and (older) the next tile have arrived; the tile after
                     // next and the next first-half operands may be in flight
                     wait_half(A1, std::integral_constant<int, 4 + MB>());
                     read_codes(0, cur ^ 4096u);           // next tile, first half
                     __builtin_amdgcn_sched_barrier(0);
-                    half(A1, apn + jstep);
+                    half(A1, apn + jstep, [] {});
                     ap = apn;
                     cur ^= 4096u;
                     --left;
