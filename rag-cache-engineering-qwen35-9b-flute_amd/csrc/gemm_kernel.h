@@ -647,6 +647,8 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                         asm volatile("s_waitcnt vmcnt(%2)" : "+v"(Aj[0]), "+v"(Aj[1])
                                      : "n"(decltype(younger)::value) : "memory");
                 };
+                // (the same in every lane: a scalar count gives a scalar loop)
+                left = __builtin_amdgcn_readfirstlane(left);
                 if (left > 0) {
                     // tile 0 is the oldest load in flight: both activation halves may stay
                     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * MB) : "memory");
@@ -657,8 +659,9 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     if (left > 1) lean_tq += qstep;
                     lean_tile(1);                         // tile 1 (or a harmless reload)
                 }
+                const int wave_hi = __builtin_amdgcn_readfirstlane(wave >> 2);
                 while (left > 0) {
-                    if ((left + (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1);
+                    if ((left + wave_hi) & 1) __builtin_amdgcn_s_setprio(1);
                     else __builtin_amdgcn_s_setprio(0);
                     const u4_t *apn = left > 1 ? ap + astep : ap;
                     // this tile's first-half operands (and, older, the tile itself) have arrived;
