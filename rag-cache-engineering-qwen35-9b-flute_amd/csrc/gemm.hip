@@ -47,16 +47,17 @@ GemmShape choose_gemm_shape(int M, int tiles, int64_t index_bytes) {
     return {4, 4, 2, 1};
 }
 
-template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false, bool DIRECT = false>
+template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false, bool DIRECT = false,
+          bool LEAN = false>
 flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
     static std::atomic<bool> attr_done{false};   // threads may race to the first call: the call is idempotent
     if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1, PERM, DIRECT>,
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_kernel<MB, KW, MW, BF16, B1, PERM, DIRECT, LEAN>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize,
                                             (int)kLdsPerCU));
         attr_done = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<MB, KW, MW, BF16, B1, PERM, DIRECT>), grid, dim3(64 * KW * MW), lds,
+    hipLaunchKernelGGL((gemm_kernel<MB, KW, MW, BF16, B1, PERM, DIRECT, LEAN>), grid, dim3(64 * KW * MW), lds,
                        stream, p);
     FLUTE_HIP_CHECK(hipGetLastError());
     return FLUTE_OK;
@@ -70,6 +71,10 @@ flute_status launch_gemm_bits(const GemmParams &p, dim3 grid, int lds, hipStream
                 if constexpr (MB == 1) {
                     if (p.rep_log2[0] == 6 && p.A8)
                         return launch_gemm<MB, KW, MW, BF16, 4, true, true>(p, grid, lds, stream);
+                }
+                if constexpr (MB == 4) {
+                    if (p.rep_log2[0] == 6 && p.lean)
+                        return launch_gemm<MB, KW, MW, BF16, 4, true, false, true>(p, grid, lds, stream);
                 }
                 if (p.rep_log2[0] == 6) return launch_gemm<MB, KW, MW, BF16, 4, true>(p, grid, lds, stream);
                 return launch_gemm<MB, KW, MW, BF16, 4>(p, grid, lds, stream);
@@ -117,9 +122,13 @@ int plan_lds(GemmParams &p, const GemmShape &shape) {
         p.tab_off[s] = lds_tables;
         lds_tables += (entries << rl) * 4;
     }
+    p.lean = 0;
     if (perm) {                                  // per-wavefront tile staging behind the tables
+        // four blocks per wavefront and one LUT group per tile: the lean loop, whose tiles go
+        // straight into two staging buffers per wavefront
+        p.lean = shape.mb == 4 && ngrp == 1 && !tuning().gemm_no_lean;
         p.stage_off = lds_tables;
-        lds_tables += shape.kw * shape.mw * 4096;
+        lds_tables += shape.kw * shape.mw * (p.lean ? 8192 : 4096);
     }
     const int slot_bytes = shape.mb * 8 * 64 * 16;
     const int lds_reduce = (shape.kw / 2) * shape.mw * slot_bytes;

@@ -26,6 +26,8 @@
 // and a ticket; the last arrival folds them in a fixed order.
 #pragma once
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace flute {
@@ -49,7 +51,8 @@ struct GemmParams {
     int bits[2];
     int tab_off[2];        // byte offset of each stream's pair tables in LDS
     int rep_log2[2];       // log2 of the table replication (lanes per entry)
-    int stage_off;         // byte offset of the per-wavefront 4 KB tile staging buffers
+    int stage_off;         // byte offset of the per-wavefront tile staging buffers (4 KB, lean loop: 8 KB)
+    int lean;              // 1: the launch uses the lean loop's instantiation
     int nstreams;
     int M, N, K, G, gs, lut_rows, R;
     int mblk_total;        // ceil(M / 16)
@@ -340,9 +343,27 @@ __device__ __forceinline__ u4_t quad_transpose(u4_t v, int lane) {
 // parameters, one or two streams.
 // DIRECT (one block per wavefront on the fast path only): the activations are read from A
 // itself and put into operand order in registers; no pre-pass launch.
-template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false, bool DIRECT = false>
+// Block mb of an activation half: 16 bytes per lane at src + mb KB, as a statement the compiler
+// does not take for a load (no wait of its own follows).
+__device__ __forceinline__ void lean_load16(u4_t &dst, const u4_t *src, int mb) {
+    switch (mb) {                                       // the offset is an immediate
+        case 0: asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(src) : "memory"); break;
+        case 1: asm volatile("global_load_dwordx4 %0, %1, off offset:1024" : "=&v"(dst) : "v"(src) : "memory"); break;
+        case 2: asm volatile("global_load_dwordx4 %0, %1, off offset:2048" : "=&v"(dst) : "v"(src) : "memory"); break;
+        default: asm volatile("global_load_dwordx4 %0, %1, off offset:3072" : "=&v"(dst) : "v"(src) : "memory"); break;
+    }
+}
+
+// LEAN (four blocks per wavefront, one 4-bit stream, one LUT group per tile): every vector memory
+// instruction of the kernel is written out and so is every wait for one.  The tile goes straight
+// into LDS (global_load_lds_dwordx4), which frees the sixteen registers a tile in flight would
+// hold; the compiler cannot count such loads next to its own (it answers one in flight with
+// vmcnt(0) in front of the next use of any loaded register), hence all or nothing.
+template <int MB, int KW, int MW, bool BF16, int B1, bool PERM = false, bool DIRECT = false,
+          bool LEAN = false>
 __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) {
     static_assert(!DIRECT || (PERM && MB == 1), "direct activations: one block, fast path");
+    static_assert(!LEAN || (PERM && !DIRECT && MB >= 2 && B1 == 4), "lean loop: fast path, operand image");
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int NT = 64 * KW * MW;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -403,7 +424,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     if constexpr (PERM) {
 #pragma unroll
         for (int gl = 0; gl < 2; ++gl) {
-            if (gl >= ngrp) break;
+            if (LEAN || gl >= ngrp) break;
             int row = p.gs >= 128 ? (t * 128) / p.gs : t * ngrp + gl;
             row = min(row, p.lut_rows - 1);
             lutv[gl] = p.lut[0][((size_t)row << 4) + (lane & 15)];
@@ -412,10 +433,55 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         // values only, not for the first tile (a conditional load here made that wait a
         // wait for everything).
         __builtin_amdgcn_sched_barrier(0);
-        load_tile();
-        load_a(A0, ap);
-        load_a(A1, ap + jstep);
+        if constexpr (!LEAN) {
+            load_tile();
+            load_a(A0, ap);
+            load_a(A1, ap + jstep);
+        }
         __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- lean loop: hand-written loads ------------------------------------------------
+    // LDS staging: two 4 KB buffers per wavefront; tile n lives in buffer n & 1.  Lane L of row i
+    // asks for the 16-byte piece that belongs at position L of that row (the same layout the
+    // register path writes: slot order and rotation of the quarters).
+    const uint32_t lds_base0 =
+        (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    const uint32_t lean_stage =
+        __builtin_amdgcn_readfirstlane(lds_base0 + p.stage_off + (uint32_t)wave * 8192u);
+    const int lean_kt = ((lane & 3) - (lane >> 4)) & 3;
+    const uint32_t lean_even = (uint32_t)((lane >> 2) * 64 + lean_kt * 16);
+    const uint32_t lean_odd = (uint32_t)(((lane >> 2) ^ 1) * 64 + lean_kt * 16);
+    const uint8_t *lean_tq = p.q[0] + ((int64_t)t * p.G + g_first) * 4096;   // wavefront-uniform
+    auto lean_tile = [&](int buf) {                    // four loads, straight into LDS
+        const uint32_t m0v = lean_stage + (uint32_t)buf * 4096u;
+        // (the pointer is the same in every lane; the compiler cannot see that through the
+        // wavefront-dependent tile count)
+        const uint64_t a64 = (uint64_t)(uintptr_t)lean_tq;
+        const uint8_t *tq_s = (const uint8_t *)(uintptr_t)(
+            (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a64) |
+            ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a64 >> 32)) << 32));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %1, %3 offset:0 nt\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:1024 nt\n\t"
+                     "global_load_lds_dwordx4 %1, %3 offset:2048 nt\n\t"
+                     "global_load_lds_dwordx4 %2, %3 offset:3072 nt"
+                     :: "s"(m0v), "v"(lean_even), "v"(lean_odd), "s"(tq_s) : "memory", "m0");
+    };
+    if constexpr (LEAN) {
+        int row = (t * 128) / p.gs;
+        row = min(row, p.lut_rows - 1);
+        const uint16_t *lp = p.lut[0] + ((size_t)row << 4) + (lane & 15);
+        uint32_t lv;
+        asm volatile("global_load_ushort %0, %1, off" : "=&v"(lv) : "v"(lp) : "memory");
+        lean_tile(0);                                  // tile 0
+        static_assert(MB == 4 || MB == 2, "operands of a half");
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) lean_load16(A0[mb], ap, mb);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) lean_load16(A1[mb], ap + jstep, mb);
+        // the LUT value is the oldest load: 4 + 2 MB younger ones may stay in flight
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(lv) : "n"(4 + 2 * MB) : "memory");
+        lutv[0] = lv;
     }
 
     // ---- pair tables ------------------------------------------------------------
@@ -511,6 +577,121 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     Q[4 * kt + 3] = v[3];
                 }
             };
+            if constexpr (LEAN) {
+                // One round = one tile of this wavefront.  Vector memory instructions of a round,
+                // in issue order: the next tile's first-half operand of the first block of rows, the
+                // tile after next (4, into the LDS buffer just read out), the other first-half
+                // operands (MB - 1, one after each block of rows of this half), the second-half
+                // operands (MB).  Blocks of rows are outermost inside a
+                // half: a block's activation operand is reloaded right after its eight
+                // products, a whole tile ahead of its use; the eight weight operands of a half
+                // stay in registers for all blocks, the last two blocks run side by side and
+                // each operand is replaced by the next half's as soon as both have used it.
+                // The products of an accumulator come in the same order as in the other loop.
+                u4_t W[8];
+                uint32_t Q8[8];
+                const uint32_t lb0 = lb[0];
+                const uint32_t rbase = lean_stage + slot * 64;
+                const int rot = rho & 3;
+                uint32_t cur = 0;                         // LDS buffer of this round's tile: 0 or 4096
+                auto read_codes = [&](int j, uint32_t boff) {
+#pragma unroll
+                    for (int kk = 0; kk < 2; ++kk) {
+                        const u4_t v = *(LdsQuad)(uintptr_t)(rbase + boff + (((2 * j + kk + rot) & 3) << 4));
+                        Q8[4 * kk + 0] = v[0];
+                        Q8[4 * kk + 1] = v[1];
+                        Q8[4 * kk + 2] = v[2];
+                        Q8[4 * kk + 3] = v[3];
+                    }
+                };
+                auto operand = [&](int o) -> u4_t {
+                    typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
+                    const int v = o >> 1, d = o & 1;
+                    u4_t w;
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4)       // q4 = ktl * 2 + s2
+                        w[q4] = *(LdsWord)__builtin_amdgcn_perm(
+                            Q8[(q4 >> 1) * 4 + v], lb0, 0x03020000u | ((4u + d * 2 + (q4 & 1)) << 8));
+                    return w;
+                };
+                // `between` runs after the first block of rows (before the pair of blocks when
+                // there are only two): work that has to follow LDS reads issued in front of the
+                // half finds them complete there instead of waiting for them
+                auto half = [&](u4_t (&Aj)[MB], const u4_t *next, auto &&between) {
+#pragma unroll
+                    for (int mb = 0; mb + 2 < MB; ++mb) {
+#pragma unroll
+                        for (int o = 0; o < 8; ++o) acc[mb][o] = mfma16<BF16>(W[o], Aj[mb], acc[mb][o]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        lean_load16(Aj[mb], next, mb);
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (mb == 0) between();
+                    }
+                    if constexpr (MB == 2) between();
+#pragma unroll
+                    for (int o = 0; o < 8; ++o) {
+                        acc[MB - 2][o] = mfma16<BF16>(W[o], Aj[MB - 2], acc[MB - 2][o]);
+                        acc[MB - 1][o] = mfma16<BF16>(W[o], Aj[MB - 1], acc[MB - 1][o]);
+                        W[o] = operand(o);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    lean_load16(Aj[MB - 2], next, MB - 2);
+                    lean_load16(Aj[MB - 1], next, MB - 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                };
+                auto wait_half = [&](u4_t (&Aj)[MB], auto younger) {
+                    if constexpr (MB == 4)
+                        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(Aj[0]), "+v"(Aj[1]), "+v"(Aj[2]), "+v"(Aj[3])
+                                     : "n"(decltype(younger)::value) : "memory");
+                    else
+                        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(Aj[0]), "+v"(Aj[1])
+                                     : "n"(decltype(younger)::value) : "memory");
+                };
+                // (the same in every lane: a scalar count gives a scalar loop)
+                left = __builtin_amdgcn_readfirstlane(left);
+                if (left > 0) {
+                    // tile 0 is the oldest load in flight: both activation halves may stay
+                    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * MB) : "memory");
+                    read_codes(0, 0);
+#pragma unroll
+                    for (int o = 0; o < 8; ++o) W[o] = operand(o);
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if (left > 1) lean_tq += qstep;
+                    lean_tile(1);                         // tile 1 (or a harmless reload)
+                }
+                const int wave_hi = __builtin_amdgcn_readfirstlane(wave >> 2);
+                while (left > 0) {
+                    if ((left + wave_hi) & 1) __builtin_amdgcn_s_setprio(1);
+                    else __builtin_amdgcn_s_setprio(0);
+                    const u4_t *apn = left > 1 ? ap + astep : ap;
+                    // this tile's first-half operands (and, older, the tile itself) have arrived;
+                    // the second-half operands may still be in flight
+                    wait_half(A0, std::integral_constant<int, MB>());
+                    read_codes(1, cur);                   // this tile, second half
+                    __builtin_amdgcn_sched_barrier(0);
+                    half(A0, apn, [&] {
+                        // the tile after next goes into the buffer just read out: not before
+                        // those reads have returned (one block of products later they have)
+                        asm volatile("s_waitcnt lgkmcnt(0)"
+                                     : "+v"(Q8[0]), "+v"(Q8[1]), "+v"(Q8[2]), "+v"(Q8[3]), "+v"(Q8[4]),
+                                       "+v"(Q8[5]), "+v"(Q8[6]), "+v"(Q8[7]) :: "memory");
+                        if (left > 2) lean_tq += qstep;
+                        lean_tile(cur != 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                    // second-half operands and (older) the next tile have arrived; the tile after
+                    // next and the next first-half operands may be in flight
+                    wait_half(A1, std::integral_constant<int, 4 + MB>());
+                    read_codes(0, cur ^ 4096u);           // next tile, first half
+                    __builtin_amdgcn_sched_barrier(0);
+                    half(A1, apn + jstep, [] {});
+                    ap = apn;
+                    cur ^= 4096u;
+                    --left;
+                }
+                // nothing may land in LDS or in a register once the tree reuses them
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            } else {
             if (left > 0) {
                 stage_write();                            // first tile, requested before the tables
                 if (left > 1) tp += qstep;
@@ -548,6 +729,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                 load_a(A1, ap + jstep);
                 __builtin_amdgcn_sched_barrier(0);
                 --left;
+            }
             }
             __builtin_amdgcn_s_setprio(0);
         } else if constexpr (B1 > 0) {
@@ -630,6 +812,9 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         }
     }
 
+    // a lean loop's loads land in LDS and registers without the compiler's knowledge: none may
+    // be in flight when the tree reuses either (wavefronts without work have issued some too)
+    if constexpr (LEAN) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // ---- tree over the KW wavefronts of one m group, through LDS ------------------
     f4_t *red = (f4_t *)smem;                           // slot = [MB*8][64] f4
     __syncthreads();                                    // tables are dead from here
