@@ -269,6 +269,21 @@ void flute_reload_tuning(void);
 int flute_workspace_decision(int64_t have_floats, int64_t need_floats, int64_t have_ints,
                              int64_t need_ints, int capturing);
 
+/*
+ * No upstream counterpart.  The library's own helper that rebuilds a 64-bit address from two
+ * 32-bit halves delivered as signed ints (the kernels move wavefront-uniform pointers into
+ * scalar registers that way), callable on the host so that it can be checked without a GPU:
+ * returns (uint32)lo | (uint32)hi << 32 for every bit pattern, bit 31 of either half included.
+ */
+uint64_t flute_join_address_halves(int32_t lo, int32_t hi);
+
+/*
+ * No upstream counterpart.  Sixteen hex digits of the SHA-256 over the sources the library was
+ * built from (csrc sources and this header, in the Makefile's order), so that a harness that
+ * loads a library by path can tell whether it is the tree's current build.
+ */
+const char *flute_build_id(void);
+
 #ifdef __cplusplus
 }
 #endif

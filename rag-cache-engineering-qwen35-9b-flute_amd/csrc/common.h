@@ -66,6 +66,14 @@ inline Segs make_segments(int K, int block) {
     return s;
 }
 
+// A 64-bit address put together from two 32-bit halves that come out of builtins returning
+// `int` (__builtin_amdgcn_readfirstlane): each half is taken as unsigned first.  Converting the
+// int straight to uint64_t sign-extends it, and a low half with bit 31 set then sets all 32 upper
+// bits of the result: an address outside every allocation.
+__host__ __device__ __forceinline__ uint64_t join_address_halves(int lo, int hi) {
+    return (uint64_t)(uint32_t)lo | ((uint64_t)(uint32_t)hi << 32);
+}
+
 // ---- 16-bit float conversions on the device --------------------------------
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));

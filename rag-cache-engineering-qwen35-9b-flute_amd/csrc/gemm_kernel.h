@@ -457,9 +457,9 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         // (the pointer is the same in every lane; the compiler cannot see that through the
         // wavefront-dependent tile count)
         const uint64_t a64 = (uint64_t)(uintptr_t)lean_tq;
-        const uint8_t *tq_s = (const uint8_t *)(uintptr_t)(
-            (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a64) |
-            ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a64 >> 32)) << 32));
+        const uint8_t *tq_s = (const uint8_t *)(uintptr_t)join_address_halves(
+            __builtin_amdgcn_readfirstlane((int)(uint32_t)a64),
+            __builtin_amdgcn_readfirstlane((int)(uint32_t)(a64 >> 32)));
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
                      "global_load_lds_dwordx4 %1, %3 offset:0 nt\n\t"
                      "global_load_lds_dwordx4 %2, %3 offset:1024 nt\n\t"

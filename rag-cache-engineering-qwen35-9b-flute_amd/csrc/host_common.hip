@@ -251,3 +251,12 @@ void flute_release_workspaces(void) {
 }
 
 }  // extern "C"
+
+extern "C" uint64_t flute_join_address_halves(int32_t lo, int32_t hi) {
+    return flute::join_address_halves(lo, hi);
+}
+
+#ifndef FLUTE_BUILD_ID
+#define FLUTE_BUILD_ID "unknown"
+#endif
+extern "C" const char *flute_build_id(void) { return FLUTE_BUILD_ID; }

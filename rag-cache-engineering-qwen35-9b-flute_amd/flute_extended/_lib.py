@@ -72,6 +72,8 @@ SYMBOLS = {
     "flute_release_workspaces": (None, []),
     "flute_reload_tuning": (None, []),
     "flute_workspace_decision": (_I, [ctypes.c_int64] * 4 + [_I]),
+    "flute_join_address_halves": (ctypes.c_uint64, [ctypes.c_int32, ctypes.c_int32]),
+    "flute_build_id": (ctypes.c_char_p, []),
 }
 
 if not os.path.exists(LIB_PATH):
@@ -85,6 +87,30 @@ for _name, (_res, _args) in SYMBOLS.items():
     _fn = getattr(lib, _name)
     _fn.restype = _res
     _fn.argtypes = _args
+
+
+def build_id() -> str:
+    """What the loaded library says it was built from (flute_build_id)."""
+    return lib.flute_build_id().decode("ascii")
+
+
+def tree_build_id() -> str:
+    """The same hash over the sources as they are in the tree now (csrc/Makefile's BUILD_ID:
+    the .hip sources in the Makefile's order, the csrc headers sorted by name, the C header).
+    Differs from build_id() when the library on disk is older than the sources."""
+    import glob
+    import hashlib
+    import re
+    csrc = os.path.join(os.path.dirname(_HERE), "csrc")
+    with open(os.path.join(csrc, "Makefile")) as f:
+        srcs = re.search(r"^SRCS := (.*)$", f.read(), re.M).group(1).split()
+    files = [os.path.join(csrc, n) for n in srcs] + sorted(glob.glob(os.path.join(csrc, "*.h")))
+    files.append(os.path.join(os.path.dirname(os.path.dirname(_HERE)), "include", "flute_hip.h"))
+    h = hashlib.sha256()
+    for name in files:
+        with open(name, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def last_error() -> str:

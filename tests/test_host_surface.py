@@ -32,6 +32,31 @@ def test_library_exports_every_declared_symbol():
     assert _lib.lib.flute_target_arch() == b"gfx950"
 
 
+@pytest.mark.parametrize("addr", [0x00007F3A80001000, 0x00007F3AFFFFF000, 0x0000800012345678,
+                                  0x00007FFF7FFFFFF0, 0xFFFFFFFE80000010, 0x0000000080000000, 0])
+def test_address_halves_rejoin_for_every_bit_pattern(addr):
+    """The kernels move wavefront-uniform 64-bit pointers into scalar registers half by half
+    through a builtin that returns a signed int.  Converting such a half straight to 64 bits
+    sign-extends it: a low half with bit 31 set then fills the upper half with ones (an address
+    outside every allocation, which small test buffers below 2 GiB of an aperture never showed).
+    The library's helper takes both halves as unsigned first; checked here on addresses with bit
+    31 set, bit 47 set, and both."""
+    as_i32 = lambda v: ctypes.c_int32(v & 0xFFFFFFFF).value        # what the builtin hands back
+    lo, hi = as_i32(addr), as_i32(addr >> 32)
+    assert _lib.lib.flute_join_address_halves(lo, hi) == addr
+    # the sign-extending form this replaces is wrong exactly when bit 31 of the low half is set
+    naive = ((lo & 0xFFFFFFFFFFFFFFFF) | ((hi & 0xFFFFFFFF) << 32)) & 0xFFFFFFFFFFFFFFFF
+    assert (naive == addr) == (lo >= 0)
+
+
+def test_loaded_library_is_the_tree_s_build():
+    """flute_build_id() is the hash of the sources the library was compiled from; a stale
+    library on disk (sources edited, `make` not run) shows up here and in any harness that
+    compares the two before timing."""
+    assert re.fullmatch(r"[0-9a-f]{16}", _lib.build_id())
+    assert _lib.build_id() == _lib.tree_build_id(), "lib/libflute_hip.so is older than csrc/: run make"
+
+
 def test_struct_layout_matches_header():
     # 9 pointers, 2 int64, 9 int32 -> 8*9 + 16 + 36 = 124, padded to 128
     assert ctypes.sizeof(_lib.FluteLinear) == 128
