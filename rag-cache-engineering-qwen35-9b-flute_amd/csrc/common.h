@@ -74,6 +74,20 @@ __host__ __device__ __forceinline__ uint64_t join_address_halves(int lo, int hi)
     return (uint64_t)(uint32_t)lo | ((uint64_t)(uint32_t)hi << 32);
 }
 
+// Reads one dword of every 64-byte line of the kernel-argument block with
+// independent scalar loads and waits for them once.  The descriptor fields are
+// then fetched through a chain of dependent scalar loads (segment -> stream ->
+// pointers); with the lines already in the scalar cache each link costs a cache
+// hit instead of a trip to L2 or memory.
+template <int BYTES>
+__device__ __forceinline__ void warm_kernargs(const void *kernargs) {
+    const uint32_t *ka = (const uint32_t *)kernargs;
+    uint32_t seen = 0;
+#pragma unroll
+    for (int o = 0; o < BYTES; o += 64) seen |= ka[o / 4];
+    asm volatile("" ::"s"(seen));
+}
+
 // ---- 16-bit float conversions on the device --------------------------------
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));

@@ -37,6 +37,37 @@ typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
 
+#ifdef FLUTE_STAMPS
+// Instrumented builds only: per-wavefront phase times (s_memrealtime, 10 ns units) and the shader
+// clock count across the K loop, written to the buffer flute_debug_stamps() was given.
+__device__ long long *g_gemm_stamps = nullptr;
+#define FLUTE_STAMP(slot)                                                                       \
+    do {                                                                                        \
+        if (g_gemm_stamps && (threadIdx.x & 63) == 0)                                           \
+            g_gemm_stamps[(((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * \
+                              (blockDim.x / 64) * 8 + (threadIdx.x >> 6) * 8 + (slot)] =        \
+                (slot) == 7 ? (long long)__builtin_readcyclecounter()                           \
+                            : (long long)__builtin_amdgcn_s_memrealtime();                      \
+    } while (0)
+#else
+#define FLUTE_STAMP(slot) do { } while (0)
+#endif
+#if defined(FLUTE_STAMPS) && FLUTE_STAMPS >= 2
+// shader cycles spent in the K loop's explicit waits, summed per wavefront (slots 4..6)
+#define FLUTE_WAIT_BEGIN() wait_t0 = (long long)__builtin_readcyclecounter()
+#define FLUTE_WAIT_END(i) wait_sum[i] += (long long)__builtin_readcyclecounter() - wait_t0
+#else
+#define FLUTE_WAIT_BEGIN() do { } while (0)
+#define FLUTE_WAIT_END(i) do { } while (0)
+#endif
+
+#ifndef FLUTE_ABL
+#define FLUTE_ABL 0
+#endif
+#ifndef FLUTE_GEMM_ORDER
+#define FLUTE_GEMM_ORDER 0
+#endif
+
 struct GemmParams {
     const uint8_t *q[2];
     const uint16_t *lut[2];
@@ -53,6 +84,7 @@ struct GemmParams {
     int rep_log2[2];       // log2 of the table replication (lanes per entry)
     int stage_off;         // byte offset of the per-wavefront tile staging buffers (4 KB, lean loop: 8 KB)
     int lean;              // 1: the launch uses the lean loop's instantiation
+    int items, units, mchunks;   // resident-grid kernel: work items = units * ksplit, units = tiles * mchunks
     int nstreams;
     int M, N, K, G, gs, lut_rows, R;
     int mblk_total;        // ceil(M / 16)
@@ -369,6 +401,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kw = wave % KW, mw = wave / KW;
     const int t = blockIdx.x;
+    FLUTE_STAMP(0);
     const int mb0 = (blockIdx.y * MW + mw) * MB;       // first 16-row block of this wavefront
     const int z = blockIdx.z;
     const int rho = lane & 15, kg = lane >> 4;
@@ -518,12 +551,17 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         }
     }
     __syncthreads();
+    FLUTE_STAMP(1);
+    FLUTE_STAMP(7);
 
     f4_t acc[MB][8];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[mb][i] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#if defined(FLUTE_STAMPS) && FLUTE_STAMPS >= 2
+    long long wait_sum[3] = {0, 0, 0}, wait_t0 = 0;
+#endif
 
     const uint32_t lds_base =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -609,15 +647,53 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     const int v = o >> 1, d = o & 1;
                     u4_t w;
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4)       // q4 = ktl * 2 + s2
-                        w[q4] = *(LdsWord)__builtin_amdgcn_perm(
+                    for (int q4 = 0; q4 < 4; ++q4) {     // q4 = ktl * 2 + s2
+#if FLUTE_ABL & 8
+                        const uint32_t addr = lb0 + (uint32_t)((o * 4 + q4) << 8);
+#else
+                        const uint32_t addr = __builtin_amdgcn_perm(
                             Q8[(q4 >> 1) * 4 + v], lb0, 0x03020000u | ((4u + d * 2 + (q4 & 1)) << 8));
+#endif
+#if FLUTE_ABL & 1
+                        w[q4] = addr;
+#else
+                        w[q4] = *(LdsWord)addr;
+#endif
+                    }
                     return w;
                 };
                 // `between` runs after the first block of rows (before the pair of blocks when
                 // there are only two): work that has to follow LDS reads issued in front of the
                 // half finds them complete there instead of waiting for them
                 auto half = [&](u4_t (&Aj)[MB], const u4_t *next, auto &&between) {
+#if FLUTE_GEMM_ORDER == 1
+                    // weight operands outermost: an operand serves all blocks of rows and is
+                    // replaced by the next half's right away, so the lookups are spread evenly
+                    // over the products (four per four)
+#pragma unroll
+                    for (int o = 0; o < 8; ++o) {
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) {
+#if FLUTE_ABL & 2
+                            asm volatile("" :: "v"(W[o]), "v"(Aj[mb]));
+#else
+                            acc[mb][o] = mfma16<BF16>(W[o], Aj[mb], acc[mb][o]);
+#endif
+                        }
+                        if (o == 0) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            between();
+                        }
+                        W[o] = operand(o);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#if !(FLUTE_ABL & 4)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) lean_load16(Aj[mb], next, mb);
+#endif
+                    __builtin_amdgcn_sched_barrier(0);
+                    return;
+#endif
 #pragma unroll
                     for (int mb = 0; mb + 2 < MB; ++mb) {
 #pragma unroll
@@ -666,22 +742,30 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     const u4_t *apn = left > 1 ? ap + astep : ap;
                     // this tile's first-half operands (and, older, the tile itself) have arrived;
                     // the second-half operands may still be in flight
+                    FLUTE_WAIT_BEGIN();
                     wait_half(A0, std::integral_constant<int, MB>());
+                    FLUTE_WAIT_END(0);
                     read_codes(1, cur);                   // this tile, second half
                     __builtin_amdgcn_sched_barrier(0);
                     half(A0, apn, [&] {
                         // the tile after next goes into the buffer just read out: not before
                         // those reads have returned (one block of products later they have)
+                        FLUTE_WAIT_BEGIN();
                         asm volatile("s_waitcnt lgkmcnt(0)"
                                      : "+v"(Q8[0]), "+v"(Q8[1]), "+v"(Q8[2]), "+v"(Q8[3]), "+v"(Q8[4]),
                                        "+v"(Q8[5]), "+v"(Q8[6]), "+v"(Q8[7]) :: "memory");
+                        FLUTE_WAIT_END(2);
                         if (left > 2) lean_tq += qstep;
+#if !(FLUTE_ABL & 4)
                         lean_tile(cur != 0);
+#endif
                         __builtin_amdgcn_sched_barrier(0);
                     });
                     // second-half operands and (older) the next tile have arrived; the tile after
                     // next and the next first-half operands may be in flight
+                    FLUTE_WAIT_BEGIN();
                     wait_half(A1, std::integral_constant<int, 4 + MB>());
+                    FLUTE_WAIT_END(1);
                     read_codes(0, cur ^ 4096u);           // next tile, first half
                     __builtin_amdgcn_sched_barrier(0);
                     half(A1, apn + jstep, [] {});
@@ -817,7 +901,15 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     if constexpr (LEAN) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // ---- tree over the KW wavefronts of one m group, through LDS ------------------
     f4_t *red = (f4_t *)smem;                           // slot = [MB*8][64] f4
+#ifdef FLUTE_STAMPS
+    if (g_gemm_stamps && lane == 0) {
+        long long *sl = g_gemm_stamps + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * (NT / 64) * 8 + wave * 8;
+        sl[7] = (long long)__builtin_readcyclecounter() - sl[7];
+    }
+#endif
+    FLUTE_STAMP(2);
     __syncthreads();                                    // tables are dead from here
+    FLUTE_STAMP(3);
 #pragma unroll
     for (int step = KW / 2; step >= 1; step >>= 1) {
         if (kw >= step && kw < 2 * step) {
@@ -838,6 +930,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
         __syncthreads();
     }
 
+    FLUTE_STAMP(4);
     // ---- totals of the workgroup as a row-major fp32 tile in LDS --------------------
     constexpr int ROWS = MW * MB * 16;                  // rows of C this workgroup owns
     constexpr int LDT = 128 + 4;                        // padded row: conflict-free both ways
@@ -854,6 +947,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     }
     __syncthreads();
 
+    FLUTE_STAMP(5);
     // Every thread now serves pieces of 8 consecutive outputs of one row: 16 threads
     // write one 256-byte row segment of C.
     constexpr int PIECES = ROWS * 16;
@@ -955,6 +1049,14 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             }
         }
     }
+#if defined(FLUTE_STAMPS) && FLUTE_STAMPS >= 2
+    if (g_gemm_stamps && lane == 0) {
+        long long *sl = g_gemm_stamps + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * (NT / 64) * 8 + wave * 8;
+        sl[4] = wait_sum[0]; sl[5] = wait_sum[1]; sl[6] = wait_sum[2];
+    }
+#else
+    FLUTE_STAMP(6);
+#endif
 }
 
 }  // namespace flute

@@ -89,21 +89,6 @@ struct GemvParams {
     int slices;             // > 0: a workgroup walks the row slices blockIdx.x, + gridDim.x, ... below this
 };
 
-// Reads one dword of every 64-byte line of the kernel-argument block with
-// independent scalar loads and waits for them once.  The descriptor fields are
-// then fetched through a chain of dependent scalar loads (segment -> stream ->
-// pointers); with the lines already in the scalar cache each link costs a cache
-// hit instead of a trip to L2 or memory.
-template <int BYTES>
-__device__ __forceinline__ void warm_kernargs(const void *kernargs) {
-    const uint32_t *ka = (const uint32_t *)kernargs;
-    uint32_t seen = 0;
-#pragma unroll
-    for (int o = 0; o < BYTES; o += 64) seen |= ka[o / 4];
-    asm volatile("" ::"s"(seen));
-}
-
-
 // ---- small device helpers ---------------------------------------------------
 
 template <int CTRL>
