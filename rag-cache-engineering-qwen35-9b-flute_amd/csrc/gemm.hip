@@ -2,7 +2,7 @@
 // pre-passes (activation permutation, residual coefficients) and the launch.
 #include <stdlib.h>
 
-#include "gemm_lean_kernel.h"
+#include "gemm_kernel.h"
 #include "host_common.h"
 
 #include <atomic>
@@ -63,23 +63,6 @@ flute_status launch_gemm(const GemmParams &p, dim3 grid, int lds, hipStream_t st
     return FLUTE_OK;
 }
 
-// The resident-grid kernel of the fast path at 64 rows and more per workgroup.
-template <int KW, int MW, bool BF16>
-flute_status launch_lean(const GemmParams &p, hipStream_t stream) {
-    static std::atomic<bool> attr_done{false};
-    if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemm_lean_kernel<KW, MW, BF16>,
-                                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                                            (int)kLdsPerCU));
-        attr_done = true;
-    }
-    const int wgs = p.items < kNumCU ? p.items : kNumCU;
-    hipLaunchKernelGGL((gemm_lean_kernel<KW, MW, BF16>), dim3(wgs), dim3(64 * KW * MW), kLeanLdsBytes,
-                       stream, p);
-    FLUTE_HIP_CHECK(hipGetLastError());
-    return FLUTE_OK;
-}
-
 template <int MB, int KW, int MW, bool BF16>
 flute_status launch_gemm_bits(const GemmParams &p, dim3 grid, int lds, hipStream_t stream) {
     if (p.nstreams == 1) {
@@ -124,7 +107,7 @@ flute_status launch_gemm_shape(const GemmShape &s, const GemmParams &p, dim3 gri
 // replication (256 bytes per entry, 64 KB per group, first table at LDS offset 0: the
 // layout the one-instruction address needs).  Everything else: as much replication as
 // the budget allows, 32 lanes at most.
-int plan_lds(GemmParams &p, const GemmShape &shape, bool allow_lean) {
+int plan_lds(GemmParams &p, const GemmShape &shape) {
     const int ngrp = p.gs >= 128 ? 1 : 128 / p.gs;
     const bool perm = p.nstreams == 1 && p.bits[0] == 4 && ngrp <= 2 &&
                       !tuning().gemm_no_perm;
@@ -143,7 +126,7 @@ int plan_lds(GemmParams &p, const GemmShape &shape, bool allow_lean) {
     if (perm) {                                  // per-wavefront tile staging behind the tables
         // four blocks per wavefront and one LUT group per tile: the lean loop, whose tiles go
         // straight into two staging buffers per wavefront
-        p.lean = allow_lean && shape.mb == 4 && ngrp == 1 && !tuning().gemm_no_lean;
+        p.lean = shape.mb == 4 && ngrp == 1 && !tuning().gemm_no_lean;
         p.stage_off = lds_tables;
         lds_tables += shape.kw * shape.mw * (p.lean ? 8192 : 4096);
     }
@@ -310,7 +293,8 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
             hipLaunchKernelGGL(gemm_prep_quad_kernel, dim3(blocks), dim3(256), 0, stream,
                                (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
                                (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
-                               rowshift);
+                               rowshift, (const uint32_t *)w->lut1,
+                               (int)(((size_t)w->lut_rows << w->b1) * 2 / 64));
         } else {
             hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
                                (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
@@ -344,23 +328,9 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
         }
         q.z_base = pass * ksplit;
         q.ztotal = passes * ksplit;
-        // (two launches that share one fold must lay their partial images out alike: the
-        // resident-grid kernel serves single launches)
-        const int lds = plan_lds(q, shape, !per_stream);
+        const int lds = plan_lds(q, shape);
         FLUTE_REQUIRE(lds <= kLdsPerCU, FLUTE_ERR_UNSUPPORTED,
                       "flute_gemm: %d bytes of LDS exceed the %d of one CU", lds, kLdsPerCU);
-        q.units = (int)units;
-        q.mchunks = mchunks;
-        q.items = (int)units * ksplit;
-        if (q.lean && !tuning().gemm_old_lean) {
-            const bool bf = w->lut_dtype == FLUTE_BF16;
-            if (shape.mw == 2)
-                st = bf ? launch_lean<4, 2, true>(q, stream) : launch_lean<4, 2, false>(q, stream);
-            else
-                st = bf ? launch_lean<8, 1, true>(q, stream) : launch_lean<8, 1, false>(q, stream);
-            if (st != FLUTE_OK) return st;
-            continue;
-        }
         st = w->lut_dtype == FLUTE_BF16 ? launch_gemm_shape<true>(shape, q, grid, lds, stream)
                                         : launch_gemm_shape<false>(shape, q, grid, lds, stream);
         if (st != FLUTE_OK) return st;

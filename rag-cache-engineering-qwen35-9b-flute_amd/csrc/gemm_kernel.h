@@ -52,22 +52,6 @@ __device__ long long *g_gemm_stamps = nullptr;
 #else
 #define FLUTE_STAMP(slot) do { } while (0)
 #endif
-#if defined(FLUTE_STAMPS) && FLUTE_STAMPS >= 2
-// shader cycles spent in the K loop's explicit waits, summed per wavefront (slots 4..6)
-#define FLUTE_WAIT_BEGIN() wait_t0 = (long long)__builtin_readcyclecounter()
-#define FLUTE_WAIT_END(i) wait_sum[i] += (long long)__builtin_readcyclecounter() - wait_t0
-#else
-#define FLUTE_WAIT_BEGIN() do { } while (0)
-#define FLUTE_WAIT_END(i) do { } while (0)
-#endif
-
-#ifndef FLUTE_ABL
-#define FLUTE_ABL 0
-#endif
-#ifndef FLUTE_GEMM_ORDER
-#define FLUTE_GEMM_ORDER 0
-#endif
-
 struct GemmParams {
     const uint8_t *q[2];
     const uint16_t *lut[2];
@@ -84,7 +68,6 @@ struct GemmParams {
     int rep_log2[2];       // log2 of the table replication (lanes per entry)
     int stage_off;         // byte offset of the per-wavefront tile staging buffers (4 KB, lean loop: 8 KB)
     int lean;              // 1: the launch uses the lean loop's instantiation
-    int items, units, mchunks;   // resident-grid kernel: work items = units * ksplit, units = tiles * mchunks
     int nstreams;
     int M, N, K, G, gs, lut_rows, R;
     int mblk_total;        // ceil(M / 16)
@@ -154,7 +137,18 @@ __device__ __forceinline__ uint32_t quad_bcast(uint32_t v) {
 __global__ void __launch_bounds__(256) gemm_prep_quad_kernel(const uint16_t *A, u4_t *Ap, int M,
                                                              int64_t lda, int G, int mblk,
                                                              int in_bf16, int out_bf16,
-                                                             const int *rowshift) {
+                                                             const int *rowshift,
+                                                             const uint32_t *warm, int warm_lines) {
+    // The launch that follows starts with a chain of dependent loads (its arguments, then the
+    // LUT rows): one thread per 64-byte line touches the LUT here, so that the rows come from
+    // the memory-side cache there instead of from memory.
+    {
+        const int line = blockIdx.x * blockDim.x + threadIdx.x;
+        if (line < warm_lines) {
+            const uint32_t seen = __builtin_nontemporal_load(warm + (size_t)line * 16);
+            asm volatile("" ::"v"(seen));
+        }
+    }
     const int segs = 2 * G;                             // 32-k segments per row
     const int64_t total = (int64_t)mblk * 16 * segs * 4;
     // the four threads of a quad share their row and their loop bound
@@ -559,9 +553,6 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[mb][i] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#if defined(FLUTE_STAMPS) && FLUTE_STAMPS >= 2
-    long long wait_sum[3] = {0, 0, 0}, wait_t0 = 0;
-#endif
 
     const uint32_t lds_base =
         (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -617,14 +608,13 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             };
             if constexpr (LEAN) {
                 // One round = one tile of this wavefront.  Vector memory instructions of a round,
-                // in issue order: the next tile's first-half operand of the first block of rows, the
-                // tile after next (4, into the LDS buffer just read out), the other first-half
-                // operands (MB - 1, one after each block of rows of this half), the second-half
-                // operands (MB).  Blocks of rows are outermost inside a
-                // half: a block's activation operand is reloaded right after its eight
-                // products, a whole tile ahead of its use; the eight weight operands of a half
-                // stay in registers for all blocks, the last two blocks run side by side and
-                // each operand is replaced by the next half's as soon as both have used it.
+                // in issue order: the tile after next (4, into the LDS buffer just read out), the
+                // next tile's first-half operands (MB), its second-half operands (MB).  Inside a
+                // half the weight operands are outermost: an operand serves all blocks of rows
+                // and is replaced by the next half's right away, so lookups and products
+                // alternate four by four (measured against blocks of rows outermost with the
+                // lookups bunched behind the last two blocks: 1 % faster; the explicit waits of
+                // either order cost no time, a wavefront's loads are there when it asks).
                 // The products of an accumulator come in the same order as in the other loop.
                 u4_t W[8];
                 uint32_t Q8[8];
@@ -647,39 +637,18 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     const int v = o >> 1, d = o & 1;
                     u4_t w;
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {     // q4 = ktl * 2 + s2
-#if FLUTE_ABL & 8
-                        const uint32_t addr = lb0 + (uint32_t)((o * 4 + q4) << 8);
-#else
-                        const uint32_t addr = __builtin_amdgcn_perm(
+                    for (int q4 = 0; q4 < 4; ++q4)       // q4 = ktl * 2 + s2
+                        w[q4] = *(LdsWord)__builtin_amdgcn_perm(
                             Q8[(q4 >> 1) * 4 + v], lb0, 0x03020000u | ((4u + d * 2 + (q4 & 1)) << 8));
-#endif
-#if FLUTE_ABL & 1
-                        w[q4] = addr;
-#else
-                        w[q4] = *(LdsWord)addr;
-#endif
-                    }
                     return w;
                 };
-                // `between` runs after the first block of rows (before the pair of blocks when
-                // there are only two): work that has to follow LDS reads issued in front of the
-                // half finds them complete there instead of waiting for them
+                // `between` runs after the first operand's products: work that has to follow LDS
+                // reads issued in front of the half finds them complete there
                 auto half = [&](u4_t (&Aj)[MB], const u4_t *next, auto &&between) {
-#if FLUTE_GEMM_ORDER == 1
-                    // weight operands outermost: an operand serves all blocks of rows and is
-                    // replaced by the next half's right away, so the lookups are spread evenly
-                    // over the products (four per four)
 #pragma unroll
                     for (int o = 0; o < 8; ++o) {
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb) {
-#if FLUTE_ABL & 2
-                            asm volatile("" :: "v"(W[o]), "v"(Aj[mb]));
-#else
-                            acc[mb][o] = mfma16<BF16>(W[o], Aj[mb], acc[mb][o]);
-#endif
-                        }
+                        for (int mb = 0; mb < MB; ++mb) acc[mb][o] = mfma16<BF16>(W[o], Aj[mb], acc[mb][o]);
                         if (o == 0) {
                             __builtin_amdgcn_sched_barrier(0);
                             between();
@@ -687,32 +656,8 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                         W[o] = operand(o);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-#if !(FLUTE_ABL & 4)
 #pragma unroll
                     for (int mb = 0; mb < MB; ++mb) lean_load16(Aj[mb], next, mb);
-#endif
-                    __builtin_amdgcn_sched_barrier(0);
-                    return;
-#endif
-#pragma unroll
-                    for (int mb = 0; mb + 2 < MB; ++mb) {
-#pragma unroll
-                        for (int o = 0; o < 8; ++o) acc[mb][o] = mfma16<BF16>(W[o], Aj[mb], acc[mb][o]);
-                        __builtin_amdgcn_sched_barrier(0);
-                        lean_load16(Aj[mb], next, mb);
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (mb == 0) between();
-                    }
-                    if constexpr (MB == 2) between();
-#pragma unroll
-                    for (int o = 0; o < 8; ++o) {
-                        acc[MB - 2][o] = mfma16<BF16>(W[o], Aj[MB - 2], acc[MB - 2][o]);
-                        acc[MB - 1][o] = mfma16<BF16>(W[o], Aj[MB - 1], acc[MB - 1][o]);
-                        W[o] = operand(o);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                    lean_load16(Aj[MB - 2], next, MB - 2);
-                    lean_load16(Aj[MB - 1], next, MB - 1);
                     __builtin_amdgcn_sched_barrier(0);
                 };
                 auto wait_half = [&](u4_t (&Aj)[MB], auto younger) {
@@ -742,30 +687,22 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
                     const u4_t *apn = left > 1 ? ap + astep : ap;
                     // this tile's first-half operands (and, older, the tile itself) have arrived;
                     // the second-half operands may still be in flight
-                    FLUTE_WAIT_BEGIN();
                     wait_half(A0, std::integral_constant<int, MB>());
-                    FLUTE_WAIT_END(0);
                     read_codes(1, cur);                   // this tile, second half
                     __builtin_amdgcn_sched_barrier(0);
                     half(A0, apn, [&] {
                         // the tile after next goes into the buffer just read out: not before
-                        // those reads have returned (one block of products later they have)
-                        FLUTE_WAIT_BEGIN();
-                        asm volatile("s_waitcnt lgkmcnt(0)"
+                        // those reads have returned (four products later they have)
+                            asm volatile("s_waitcnt lgkmcnt(0)"
                                      : "+v"(Q8[0]), "+v"(Q8[1]), "+v"(Q8[2]), "+v"(Q8[3]), "+v"(Q8[4]),
                                        "+v"(Q8[5]), "+v"(Q8[6]), "+v"(Q8[7]) :: "memory");
-                        FLUTE_WAIT_END(2);
                         if (left > 2) lean_tq += qstep;
-#if !(FLUTE_ABL & 4)
                         lean_tile(cur != 0);
-#endif
                         __builtin_amdgcn_sched_barrier(0);
                     });
                     // second-half operands and (older) the next tile have arrived; the tile after
                     // next and the next first-half operands may be in flight
-                    FLUTE_WAIT_BEGIN();
                     wait_half(A1, std::integral_constant<int, 4 + MB>());
-                    FLUTE_WAIT_END(1);
                     read_codes(0, cur ^ 4096u);           // next tile, first half
                     __builtin_amdgcn_sched_barrier(0);
                     half(A1, apn + jstep, [] {});
@@ -1049,14 +986,7 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
             }
         }
     }
-#if defined(FLUTE_STAMPS) && FLUTE_STAMPS >= 2
-    if (g_gemm_stamps && lane == 0) {
-        long long *sl = g_gemm_stamps + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * (NT / 64) * 8 + wave * 8;
-        sl[4] = wait_sum[0]; sl[5] = wait_sum[1]; sl[6] = wait_sum[2];
-    }
-#else
     FLUTE_STAMP(6);
-#endif
 }
 
 }  // namespace flute

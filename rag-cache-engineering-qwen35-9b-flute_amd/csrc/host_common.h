@@ -34,7 +34,7 @@ int workspace_decision(size_t have_floats, size_t need_floats, size_t have_ints,
 // gemv4_walk = -1 (the launcher's own choice).
 struct Tuning {
     int gemv_rw, gemv_waves, gemv_table_log2, gemv_prerotate, gemv4_pf, gemv_no_fast, gemv4_walk;
-    int gemm_rows, gemm_no_perm, gemm_ksplit, gemm_no_direct, gemm_no_lean, gemm_old_lean;
+    int gemm_rows, gemm_no_perm, gemm_ksplit, gemm_no_direct, gemm_no_lean;
     int fht_steps;
 };
 const Tuning &tuning();
