@@ -49,6 +49,8 @@ extern "C" flute_status flute_dequant(const flute_linear *w, int which, void *W_
     flute_status st = validate_linear(w, 1, "flute_dequant");
     if (st != FLUTE_OK) return st;
     FLUTE_REQUIRE(W_out != nullptr, FLUTE_ERR_INVALID, "flute_dequant: output is NULL");
+    FLUTE_REQUIRE(((uintptr_t)W_out & 3) == 0, FLUTE_ERR_INVALID,
+                  "flute_dequant: output must be 4-byte aligned (two weights per store)");
     FLUTE_REQUIRE(which == 1 || (which == 2 && w->b2 > 0), FLUTE_ERR_INVALID,
                   "flute_dequant: stream %d is not present", which);
     const uint8_t *q = (const uint8_t *)(which == 1 ? w->q1 : w->q2);

@@ -148,6 +148,8 @@ extern "C" flute_status flute_embedding(const flute_linear *w, const int64_t *id
     FLUTE_REQUIRE(w->bias == nullptr, FLUTE_ERR_INVALID, "flute_embedding: an embedding has no bias");
     FLUTE_REQUIRE(w->awq == nullptr, FLUTE_ERR_INVALID,
                   "flute_embedding: an embedding table carries no activation scale");
+    FLUTE_REQUIRE(((uintptr_t)ids & 7) == 0, FLUTE_ERR_INVALID,
+                  "flute_embedding: ids are int64 and must be 8-byte aligned");
     FLUTE_REQUIRE(((uintptr_t)out & 3) == 0, FLUTE_ERR_INVALID,
                   "flute_embedding: out must be 4-byte aligned");
     EmbParams p = {};

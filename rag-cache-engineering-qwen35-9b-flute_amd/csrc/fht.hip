@@ -472,6 +472,13 @@ extern "C" flute_status flute_fht(const void *x, const float *signs, const float
     FLUTE_REQUIRE(dtype == FLUTE_F16 || dtype == FLUTE_BF16 || dtype == FLUTE_F32, FLUTE_ERR_INVALID,
                   "flute_fht: dtype must be float16, bfloat16 or float32");
     FLUTE_REQUIRE(M >= 0, FLUTE_ERR_INVALID, "flute_fht: M must be >= 0");
+    {
+        const uintptr_t elem = dtype == FLUTE_F32 ? 3 : 1;
+        FLUTE_REQUIRE(((uintptr_t)x & elem) == 0 && ((uintptr_t)out & elem) == 0, FLUTE_ERR_INVALID,
+                      "flute_fht: x and out must be aligned to their element size");
+        FLUTE_REQUIRE(((uintptr_t)signs & 3) == 0 && ((uintptr_t)awq & 3) == 0, FLUTE_ERR_INVALID,
+                      "flute_fht: signs and awq are fp32 and must be 4-byte aligned");
+    }
     FLUTE_REQUIRE(K >= 32 && K % 32 == 0 && K <= 65504, FLUTE_ERR_INVALID,
                   "flute_fht: K must be a multiple of 32 in [32, 65504] (got %d)", K);
     FLUTE_REQUIRE(!(awq && adjoint), FLUTE_ERR_INVALID,

@@ -335,6 +335,7 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
                                         : launch_gemm_shape<false>(shape, q, grid, lds, stream);
         if (st != FLUTE_OK) return st;
     }
+    workspace_done(stream);
     return FLUTE_OK;
 }
 

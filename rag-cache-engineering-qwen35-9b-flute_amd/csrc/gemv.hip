@@ -107,12 +107,16 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     FLUTE_REQUIRE(count >= 1 && count <= kGemvMaxSegs, FLUTE_ERR_INVALID,
                   "%s: 1..%d weights per launch (got %d)", who, kGemvMaxSegs, count);
     FLUTE_REQUIRE(x != nullptr, FLUTE_ERR_INVALID, "%s: x is NULL", who);
+    FLUTE_REQUIRE(((uintptr_t)x & 15) == 0, FLUTE_ERR_INVALID,
+                  "%s: x must be 16-byte aligned (the kernels read it 16 bytes at a time)", who);
     FLUTE_REQUIRE(act_dtype == FLUTE_F16 || act_dtype == FLUTE_BF16, FLUTE_ERR_INVALID,
                   "%s: activations must be float16 or bfloat16", who);
     for (int i = 0; i < count; ++i) {
         flute_status st = validate_linear(&segs[i], 0, who);
         if (st != FLUTE_OK) return st;
         FLUTE_REQUIRE(outs[i] != nullptr, FLUTE_ERR_INVALID, "%s: output %d is NULL", who, i);
+        FLUTE_REQUIRE(((uintptr_t)outs[i] & 1) == 0, FLUTE_ERR_INVALID,
+                      "%s: output %d must be 2-byte aligned", who, i);
         FLUTE_REQUIRE(segs[i].K == segs[0].K, FLUTE_ERR_INVALID,
                       "%s: all weights of one launch must share K (%d vs %d)", who, segs[i].K,
                       segs[0].K);
@@ -143,7 +147,9 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     int rw, waves;
     bool rotated = false;
     for (int i = 0; i < count; ++i) rotated |= segs[i].signs != nullptr;
-    choose_shape(rows, G, split, &rw, &split, &waves, !rotated);
+    // (the library's own K split was measured on single weights only: merged gate/up launches
+    // split when the caller asks for it)
+    choose_shape(rows, G, split, &rw, &split, &waves, !rotated && !silu_mul);
     FLUTE_REQUIRE((G / split) % (32 / rw) == 0, FLUTE_ERR_UNSUPPORTED,
                   "%s: K/64/split = %d is not a whole number of wavefront loads", who, G / split);
     const int gs_tiles = G / split;
@@ -461,7 +467,9 @@ flute_status launch(Plan &plan, int act_dtype, hipStream_t stream, float *fixed_
             }
         }
     }
-    return plan.lut_bf16 ? launch_width<true>(plan, stream) : launch_width<false>(plan, stream);
+    const flute_status st = plan.lut_bf16 ? launch_width<true>(plan, stream) : launch_width<false>(plan, stream);
+    if ((plan.p_floats || plan.npre) && !fixed_base) workspace_done(stream);
+    return st;
 }
 
 // ---- the allocation-free variant's scratch ------------------------------------------
@@ -485,13 +493,20 @@ static unsigned char *g_scratch_ptr[kMaxDevices] = {};
 
 // Device address of this device's copy of the array (the array's name is a host-side
 // stand-in, not a device address): resolved once per device, with that device current.
-flute_status noalloc_scratch(unsigned char **out) {
+flute_status noalloc_scratch(unsigned char **out, hipStream_t stream) {
     int dev = 0;
     FLUTE_HIP_CHECK(hipGetDevice(&dev));
     FLUTE_REQUIRE(dev >= 0 && dev < kMaxDevices, FLUTE_ERR_UNSUPPORTED,
                   "flute_gemv_noalloc: device ordinal %d beyond %d", dev, kMaxDevices);
     std::lock_guard<std::mutex> guard(g_scratch_mu);
     if (!g_scratch_ptr[dev]) {
+        // resolving the symbol may load the code object: not something to do inside a capture
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        FLUTE_HIP_CHECK(hipStreamIsCapturing(stream, &cap));
+        FLUTE_REQUIRE(cap == hipStreamCaptureStatusNone, FLUTE_ERR_INVALID,
+                      "flute_gemv_noalloc: the first call on device %d that needs the scratch array "
+                      "resolves its address and must not be under stream capture; make one such "
+                      "call outside the capture first", dev);
         unsigned char *ptr = nullptr;
         FLUTE_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
         FLUTE_REQUIRE(ptr != nullptr, FLUTE_ERR_HIP,
@@ -535,7 +550,7 @@ flute_status flute_gemv_noalloc(const flute_linear *w, const void *x, void *y, i
                   kNoAllocTickets, w->N, w->K, w->R, plan.p.split);
     if (need.floats == 0) return launch(plan, act_dtype, (hipStream_t)stream);
     unsigned char *ptr = nullptr;
-    st = noalloc_scratch(&ptr);
+    st = noalloc_scratch(&ptr, (hipStream_t)stream);
     if (st != FLUTE_OK) return st;
     int *tickets = (int *)ptr;
     float *base = (float *)(ptr + kNoAllocTickets * sizeof(int));
@@ -591,9 +606,9 @@ int flute_pick_split(int N, int K) {
 
 int64_t flute_gemv_lds_bytes(const flute_linear *w, int split) {
     Plan plan;
-    char dummy_x = 0, dummy_y = 0;
-    void *outs[1] = {&dummy_y};
-    if (make_plan(w, 1, &dummy_x, outs, (w && w->lut_dtype == FLUTE_BF16) ? FLUTE_BF16 : FLUTE_F16,
+    alignas(16) char dummy_x[16] = {}, dummy_y[16] = {};    // never dereferenced
+    void *outs[1] = {dummy_y};
+    if (make_plan(w, 1, dummy_x, outs, (w && w->lut_dtype == FLUTE_BF16) ? FLUTE_BF16 : FLUTE_F16,
                   split, 0, "flute_gemv_lds_bytes", &plan) != FLUTE_OK)
         return 0;
     return (int64_t)plan.lds_bytes;

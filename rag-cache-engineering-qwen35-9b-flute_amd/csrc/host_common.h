@@ -20,6 +20,9 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who);
 // part of a capture.  Warm the shape up outside the capture first.
 flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float **P,
                            int **tickets);
+// Called by an entry point after the last launch that uses the workspace: once the workspace
+// has been used from two streams, records the event the next stream's call waits on.
+void workspace_done(hipStream_t stream);
 
 // What get_workspace does for a request, as pure host arithmetic: 0 = the buffers are
 // large enough, 1 = they grow, 2 = growth refused because the stream is capturing.

@@ -61,6 +61,15 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who) {
         FLUTE_REQUIRE(aligned(w->q2, 16), FLUTE_ERR_INVALID,
                       "%s: stream-2 indices must be 16-byte aligned", who);
     }
+    // Operands the kernels read element by element still have to sit on an element boundary
+    // (16-bit values on 2 bytes, fp32 on 4): an odd address is refused here rather than met
+    // by a load in the kernel.
+    FLUTE_REQUIRE(w->b2 == 0 || aligned(w->lut2, 2), FLUTE_ERR_INVALID, "%s: lut2 misaligned", who);
+    FLUTE_REQUIRE(aligned(w->resA, 2) && aligned(w->resB, 2), FLUTE_ERR_INVALID,
+                  "%s: resA and resB must be 2-byte aligned", who);
+    FLUTE_REQUIRE(aligned(w->bias, 2), FLUTE_ERR_INVALID, "%s: bias must be 2-byte aligned", who);
+    FLUTE_REQUIRE(aligned(w->signs, 4) && aligned(w->awq, 4), FLUTE_ERR_INVALID,
+                  "%s: rotation signs and awq scale are fp32 and must be 4-byte aligned", who);
     FLUTE_REQUIRE((w->resA != nullptr) == (w->resB != nullptr), FLUTE_ERR_INVALID,
                   "%s: resB and resA must be supplied together", who);
     FLUTE_REQUIRE((w->resA != nullptr) == (w->R > 0), FLUTE_ERR_INVALID,
@@ -85,10 +94,14 @@ struct Workspace {
     int *tickets = nullptr;
     size_t floats = 0;
     size_t ints = 0;
-    // the stream of the last call that took the workspace, and an event to order the next
-    // stream behind it
+    // The stream of the last call that took the workspace (compared, never dereferenced: the
+    // caller may have destroyed it since), and the event that call recorded behind its launches
+    // for a call on another stream to wait on.  Events are only recorded once a second stream
+    // has been seen (`shared`), so single-stream use pays nothing.
     hipStream_t last_stream = nullptr;
     bool used = false;
+    bool shared = false;
+    bool recorded = false;
     hipEvent_t handover = nullptr;
 };
 
@@ -146,31 +159,47 @@ flute_status get_workspace(size_t floats, size_t ints, hipStream_t stream, float
         ws.ints = want;
     }
     // One workspace serves every stream of the device.  A call on another stream than the last
-    // one is ordered behind it with an event, so that two eager streams cannot overwrite each
-    // other's partial sums; calls that really overlap (issued from two host threads at once)
-    // and streams under capture (an event of a foreign stream cannot join a capture) remain
-    // the caller's to order.
+    // one is ordered behind it: it waits on the event the earlier call recorded at its end
+    // (workspace_done).  The earlier stream's handle is not touched (it may be gone).  The first
+    // change of stream finds no event yet and waits for the device once.  Calls that really
+    // overlap (two host threads at once) and streams under capture (an event recorded outside
+    // a capture cannot join it) remain the caller's to order.
     if (ws.used && ws.last_stream != stream) {
-        hipStreamCaptureStatus mine = hipStreamCaptureStatusNone, theirs = hipStreamCaptureStatusNone;
+        hipStreamCaptureStatus mine = hipStreamCaptureStatusNone;
         FLUTE_HIP_CHECK(hipStreamIsCapturing(stream, &mine));
-        // the earlier stream may be gone by now (its work is then complete): a failing query
-        // means there is nothing to wait for
-        const bool alive = hipStreamIsCapturing(ws.last_stream, &theirs) == hipSuccess;
-        if (!alive) (void)hipGetLastError();
-        if (alive && mine == hipStreamCaptureStatusNone && theirs == hipStreamCaptureStatusNone) {
-            if (!ws.handover)
-                FLUTE_HIP_CHECK(hipEventCreateWithFlags(&ws.handover, hipEventDisableTiming));
-            if (hipEventRecord(ws.handover, ws.last_stream) == hipSuccess)
+        if (mine == hipStreamCaptureStatusNone) {
+            if (ws.recorded)
                 FLUTE_HIP_CHECK(hipStreamWaitEvent(stream, ws.handover, 0));
             else
-                (void)hipGetLastError();
+                FLUTE_HIP_CHECK(hipDeviceSynchronize());
         }
+        ws.shared = true;
     }
     ws.last_stream = stream;
     ws.used = true;
     *P = ws.P;
     *tickets = ws.tickets;
     return FLUTE_OK;
+}
+
+void workspace_done(hipStream_t stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> guard(g_ws_mu);
+    auto it = g_ws.find(dev);
+    if (it == g_ws.end() || !it->second.shared) return;
+    Workspace &ws = it->second;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        ws.recorded = false;       // nothing a later stream could wait on: it synchronises instead
+        return;
+    }
+    if (!ws.handover && hipEventCreateWithFlags(&ws.handover, hipEventDisableTiming) != hipSuccess) {
+        ws.handover = nullptr;
+        ws.recorded = false;
+        return;
+    }
+    ws.recorded = hipEventRecord(ws.handover, stream) == hipSuccess;
 }
 
 static Tuning g_tuning;

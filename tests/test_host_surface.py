@@ -95,6 +95,16 @@ def _desc(N=256, K=128, b1=4, b2=0, gs=128, R=0, **over):
     ({"resA": 4096}, _lib.FLUTE_ERR_INVALID),             # resA without resB
     ({"awq": 4096}, _lib.FLUTE_ERR_INVALID),              # awq without signs
     ({"lut_dtype": 2}, _lib.FLUTE_ERR_INVALID),
+    # operands off their element boundary: one case per pointer the kernels read
+    ({"lut1": 4097}, _lib.FLUTE_ERR_INVALID),
+    ({"b2": 2, "lut2": 4097}, _lib.FLUTE_ERR_INVALID),
+    ({"b2": 2, "q2": 4104}, _lib.FLUTE_ERR_INVALID),      # stream-2 indices 8- but not 16-byte aligned
+    ({"R": 8, "resA": 4097, "resB": 4096}, _lib.FLUTE_ERR_INVALID),
+    ({"R": 8, "resA": 4096, "resB": 4099}, _lib.FLUTE_ERR_INVALID),
+    ({"bias": 4097}, _lib.FLUTE_ERR_INVALID),
+    ({"signs": 4098}, _lib.FLUTE_ERR_INVALID),
+    ({"signs": 4096, "awq": 4102}, _lib.FLUTE_ERR_INVALID),
+    ({"signs": 4096, "awq": 4100, "bias": 4098, "R": 8, "resA": 4098, "resB": 4102}, _lib.FLUTE_OK),
 ])
 def test_c_validation(over, code):
     w = _desc(**over)
@@ -115,6 +125,18 @@ def test_c_entry_points_refuse_before_touching_the_device():
     assert _lib.lib.flute_fht(4096, 4096, 4096, 4096, 1, 128, 0, 1, 0, None) == _lib.FLUTE_ERR_INVALID
     assert _lib.lib.flute_fht(4096, 4096, None, 4096, 1, 32768, 0, 0, 0, None) \
         == _lib.FLUTE_ERR_UNSUPPORTED
+    # operands of the calls themselves: x is read 16 bytes at a time, outputs are 16-bit stores,
+    # the rotation's rows sit on element boundaries, the dense output takes 4-byte stores
+    assert _lib.lib.flute_gemv(ctypes.byref(w), 4096 + 8, 4096, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert "16-byte" in _lib.last_error()
+    assert _lib.lib.flute_gemv(ctypes.byref(w), 4096, 4097, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_gemv_noalloc(ctypes.byref(w), 4096 + 2, 4096, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_fht(4097, 4096, None, 4096, 1, 128, 0, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_fht(4096, 4098, None, 4096, 1, 128, 0, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_fht(4098, 4096, None, 4096, 1, 128, _lib.F32, 0, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_dequant(ctypes.byref(w), 1, 4098, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_gemm(ctypes.byref(w), 4097, 4096, 4, 128, 256, 0, None) == _lib.FLUTE_ERR_INVALID
+    assert _lib.lib.flute_embedding(ctypes.byref(w), 4100, 1, 4096, None) == _lib.FLUTE_ERR_INVALID
     g, u = _desc(), _desc(N=384)
     assert _lib.lib.flute_gemv_mlp(ctypes.byref(g), ctypes.byref(u), 4096, 4096, 0, 0, None) \
         == _lib.FLUTE_ERR_INVALID
