@@ -334,6 +334,130 @@ def load_tied_pair(lm_head_meta: Dict, embed_meta: Optional[Dict], artifacts_dir
 _HEADS = ("model.lm_head.weight", "model.embed_tokens.weight")
 
 
+def read_norm_gain_doc(artifacts_dir: str) -> Optional[Dict]:
+    """norm_gain_edits.json of an artifact directory, or None when the set has none
+    (scripts/palettized_modules.py:3122-3129 upstream)."""
+    import json
+    path = os.path.join(artifacts_dir, "norm_gain_edits.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        return json.load(f)
+
+
+def _load_vector(path: str, what: str) -> torch.Tensor:
+    try:
+        arr = np.load(path, allow_pickle=False)
+    except Exception as exc:
+        raise ValueError(f"{what}: cannot read {path!r} ({exc})") from exc
+    return torch.from_numpy(np.ascontiguousarray(arr))
+
+
+def recover_awq_scales(model, artifacts_dir: str, metadata: Dict, norm_doc: Optional[Dict],
+                       verify_sha: bool = True) -> Dict:
+    """Per-channel AWQ scales of every norm group with alpha > 0, keyed by consumer tensor
+    name: what PalettizedLinear(awq_scale=...) needs to compensate sets whose rotation was
+    folded before the AWQ scale (scripts/palettized_modules.py:3130-3262 upstream).
+
+    Must run on the PRISTINE model, before apply_norm_gain_edits.  The producer folded the
+    inverse scale into the zero-centred RMSNorm gain exactly, w' = (1 + w)/s - 1, and stored
+    the complete edited parameter, so s = (1 + w_model) / (1 + w_edited) per channel.  An
+    entry that pins the scale itself ("awq_scale_file", written by exports whose gain was
+    trained further) is preferred over that quotient.
+
+    Refused loudly, never served approximately:
+      * an edited gain with 1 + w' < 0 anywhere (the legacy w/s fold, not a zero-centred one);
+      * scales that are not finite or leave (0, 1 + 2e-3];
+      * a consumer whose own metadata records AWQ statistics (s_min / s_max / s_mean) more
+        than 2 % away from the recovered ones;
+      * shapes that do not match the model's parameter; a parameter the model does not have.
+    Returns {} when there are no edits or none with alpha > 0."""
+    edits = (norm_doc or {}).get("edits") or {}
+    if not edits:
+        return {}
+    params = dict(model.named_parameters())
+    tensors_meta = metadata.get("tensors") or {}
+    scales: Dict = {}
+    for pname, entry in edits.items():
+        try:
+            alpha = float(entry.get("alpha") or 0.0)
+        except (TypeError, ValueError):
+            alpha = 0.0
+        if alpha <= 0.0:
+            continue
+        what = f"awq_recover:{pname}"
+        if pname not in params:
+            raise KeyError(f"{what}: the model has no such parameter (norm edit with "
+                           f"alpha={alpha}): artifact set and model disagree")
+        w_model = params[pname].detach().float().cpu()
+        pinned = entry.get("awq_scale_file")
+        if pinned:
+            path = os.path.join(artifacts_dir, str(pinned))
+            _check_sha(path, entry.get("awq_scale_sha256"), what, verify_sha)
+            s = _load_vector(path, what).float().reshape(-1)
+            if s.numel() != w_model.numel():
+                raise ValueError(f"{what}: pinned scale has {s.numel()} entries, the norm "
+                                 f"parameter {w_model.numel()}")
+        else:
+            path = os.path.join(artifacts_dir, entry["file"])
+            _check_sha(path, entry.get("sha256"), what, verify_sha)
+            w_edit = _load_vector(path, what).float()
+            if tuple(w_edit.shape) != tuple(w_model.shape):
+                raise ValueError(f"{what}: edited gain has shape {tuple(w_edit.shape)}, the "
+                                 f"model's parameter {tuple(w_model.shape)}")
+            gain = 1.0 + w_edit
+            if bool((gain < 0).any()):
+                raise ValueError(f"{what}: 1 + w_edited is negative somewhere: not a fold into a "
+                                 f"zero-centred RMSNorm gain (a legacy w/s producer?); no "
+                                 f"compensation is derived from it")
+            s = ((1.0 + w_model) / gain.clamp(min=1e-6)).reshape(-1)
+        if not bool(torch.isfinite(s).all()) or bool((s <= 0).any()) or float(s.max()) > 1.0 + 2e-3:
+            raise ValueError(f"{what}: recovered scales leave (0, 1]: min {float(s.min()):.4g}, "
+                             f"max {float(s.max()):.4g}; norm edit and checkpoint disagree")
+        stats = {"s_min": float(s.min()), "s_max": float(s.max()), "s_mean": float(s.mean())}
+        for consumer in entry.get("consumers") or []:
+            cname = str(consumer)
+            recorded = (tensors_meta.get(cname) or {}).get("awq") or {}
+            if recorded.get("applied"):
+                for key, got in stats.items():
+                    want = recorded.get(key)
+                    if want is not None and abs(got - float(want)) > 0.02 * max(1.0, abs(float(want))):
+                        raise ValueError(f"awq_recover:{cname}: recovered {key}={got:.4g}, the "
+                                         f"tensor's metadata says {float(want):.4g} (> 2 %): the "
+                                         f"norm edits and the tensor describe different scales")
+            scales.setdefault(cname, s)
+    return scales
+
+
+def apply_norm_gain_edits(model, artifacts_dir: str, verify_sha: bool = True,
+                          strict: bool = True) -> Dict:
+    """Copies every edited RMSNorm gain of norm_gain_edits.json (norm_edits/*.npy, each the
+    COMPLETE edited parameter) into the parameter it names, cast to that parameter's dtype;
+    after constructing the model, before the module swap.  Idempotent.  Returns the entries
+    applied (scripts/palettized_modules.py:3029-3077 upstream)."""
+    doc = read_norm_gain_doc(artifacts_dir)
+    if not doc:
+        return {}
+    params = dict(model.named_parameters())
+    applied = {}
+    for pname, entry in (doc.get("edits") or {}).items():
+        if pname not in params:
+            if strict:
+                raise KeyError(f"apply_norm_gain_edits: parameter {pname!r} not found in model")
+            continue
+        path = os.path.join(artifacts_dir, entry["file"])
+        _check_sha(path, entry.get("sha256"), f"norm_edit:{pname}", verify_sha)
+        value = _load_vector(path, f"norm_edit:{pname}")
+        target = params[pname]
+        if tuple(value.shape) != tuple(target.shape):
+            raise ValueError(f"norm_edit:{pname}: shape {tuple(value.shape)} != parameter shape "
+                             f"{tuple(target.shape)}")
+        with torch.no_grad():
+            target.copy_(value.to(target.dtype))
+        applied[pname] = entry
+    return applied
+
+
 def load_metadata(artifacts_dir: str) -> Dict:
     """metadata.json of an artifact directory (upstream :3114-3117)."""
     import json

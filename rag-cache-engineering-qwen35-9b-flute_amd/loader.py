@@ -39,7 +39,7 @@ def set_forward_mode(model, forward: str = "kernel", fuse_mlp: bool = True):
 
 def load_quant_model(artifacts_dir, model_name, device, residual=False, dtype=None,
                      forward="kernel", awq_compensation=True, heads_dir=None, model=None,
-                     awq_scales=None, verify_sha=True, **unused):
+                     awq_scales=None, verify_sha=True, apply_norm_edits=True, **unused):
     """Returns (model, metadata), like upstream's loader.
 
     model: the constructed torch model whose layers are to be swapped.  Required: without
@@ -48,9 +48,14 @@ def load_quant_model(artifacts_dir, model_name, device, residual=False, dtype=No
     metadata returned.
     forward: "kernel" or "reference".  residual: attach the low-rank residual pairs.
     dtype: dtype of the modules that stay dense (default float16); palettized buffers keep
-    their own types.  awq_scales: consumer name -> (K,) scale map (upstream recovers it from
-    norm_gain_edits.json on the pristine model; here the caller passes it);
-    awq_compensation=False drops it.  heads_dir: separate artifact directory of the
+    their own types.  With apply_norm_edits (default), the artifact set's norm_gain_edits.json is
+    honoured as upstream does (scripts/palettized_modules.py:3378-3386): while the model is
+    still pristine the AWQ scales of every alpha > 0 norm group are recovered from the edits
+    (artifacts.recover_awq_scales), then the edited gains are copied into the model
+    (artifacts.apply_norm_gain_edits), then the layers are swapped with those scales.
+    awq_scales: a consumer name -> (K,) scale map of the caller's own takes the place of the
+    recovered one; awq_compensation=False drops the compensation (differential debugging:
+    the rotate-then-scale sets then serve wrong values on purpose).  heads_dir: separate artifact directory of the
     embedding and lm_head records.  Keyword arguments of upstream's memory attachments
     (use_m1m2, m1m2_mem_size, m1m2_gates_path) are accepted and ignored: those modules are
     not part of this package."""
@@ -68,6 +73,13 @@ def load_quant_model(artifacts_dir, model_name, device, residual=False, dtype=No
         raise TypeError(f"load_quant_model: unexpected arguments {sorted(extra)}")
     metadata = artifacts.load_metadata(artifacts_dir)
     model = model.to(dtype if dtype is not None else torch.float16)
+    if apply_norm_edits:
+        norm_doc = artifacts.read_norm_gain_doc(artifacts_dir)
+        if norm_doc and awq_compensation and awq_scales is None:
+            # on the pristine gains: the recovery divides them by the edited ones
+            awq_scales = artifacts.recover_awq_scales(model, artifacts_dir, metadata, norm_doc,
+                                                      verify_sha=verify_sha)
+        artifacts.apply_norm_gain_edits(model, artifacts_dir, verify_sha=verify_sha)
     artifacts.replace_linear_with_palettized(
         model, metadata, artifacts_dir, residual=residual, reference=(forward == "reference"),
         verify_sha=verify_sha, awq_scales=awq_scales if awq_compensation else None,

@@ -168,3 +168,185 @@ def test_load_quant_model_kernel_mode_matches_reference_mode(tmp_path, dtype):
     loader.set_forward_mode(ker_model, "reference")
     assert rel_l2(ker_model(ids.to("cuda:0")).float().cpu(), ref_model(ids)) <= \
         (2e-3 if dtype == torch.float16 else 1.5e-2)
+
+
+# ---- norm-gain edits and the AWQ scales recovered from them ---------------------------------
+# (scripts/palettized_modules.py:3029-3077, 3130-3262, 3378-3386 upstream)
+
+def _sha_of(path):
+    import hashlib
+    with open(path, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
+def _awq_artifact_dir(tmp, pinned=False, legacy=False, stats_off=False):
+    """The two-layer set above with a rotation on layer 0's gate/up, an AWQ scale folded into
+    layer 0's norm gain the zero-centred way (w' = (1 + w)/s - 1) and the edit files that
+    record it.  Returns (weights, model with the pristine gain, the scale)."""
+    import numpy as np
+    weights = _artifact_dir(tmp)
+    meta = artifacts.load_metadata(tmp)
+    g = torch.Generator().manual_seed(5)
+    s = (torch.rand(H, generator=g) * 0.7 + 0.3).float()                # (0.3, 1]
+    torch.manual_seed(1)
+    model = _LM()
+    with torch.no_grad():
+        model.model.layers[0].norm.weight.copy_(torch.randn(H, generator=g) * 0.1)
+    w0 = model.model.layers[0].norm.weight.detach().float()
+    edited = (w0 / s) if legacy else ((1.0 + w0) / s - 1.0)
+    if legacy:
+        edited = edited - 2.0                                             # 1 + w' < 0: not a gain fold
+    os.makedirs(os.path.join(tmp, "norm_edits"), exist_ok=True)
+    np.save(os.path.join(tmp, "norm_edits", "l0.npy"), edited.numpy())
+    # (a consumer is named by its key in metadata["tensors"], which is also its "var")
+    consumers = ["model.layers.0.mlp.gate_proj.weight", "model.layers.0.mlp.up_proj.weight"]
+    entry = {"file": "norm_edits/l0.npy", "sha256": _sha_of(os.path.join(tmp, "norm_edits", "l0.npy")),
+             "alpha": 0.5, "consumers": consumers}
+    if pinned:
+        np.save(os.path.join(tmp, "norm_edits", "l0_scale.npy"), s.numpy())
+        entry["awq_scale_file"] = "norm_edits/l0_scale.npy"
+        entry["awq_scale_sha256"] = _sha_of(os.path.join(tmp, "norm_edits", "l0_scale.npy"))
+    doc = {"edits": {"model.layers.0.norm.weight": entry,
+                     "model.layers.1.norm.weight": {"file": "norm_edits/l0.npy", "alpha": 0.0,
+                                                    "consumers": []}}}
+    with open(os.path.join(tmp, "norm_gain_edits.json"), "w") as f:
+        json.dump(doc, f)
+    for key in ("model.layers.0.mlp.gate_proj.weight", "model.layers.0.mlp.up_proj.weight"):
+        rec = meta["tensors"][key]
+        rec["var"] = key
+        rec["rotation"] = {"seed": 3, "k": H}
+        off = 0.2 if stats_off else 0.0
+        rec["awq"] = {"applied": True, "fold_order": "rotate_then_awq", "s_min": float(s.min()) + off,
+                      "s_max": float(s.max()), "s_mean": float(s.mean())}
+    with open(os.path.join(tmp, "metadata.json"), "w") as f:
+        json.dump(meta, f)
+    return weights, model, s
+
+
+@pytest.mark.parametrize("pinned", [False, True])
+def test_awq_scales_are_recovered_from_the_norm_edits(tmp_path, pinned):
+    tmp = str(tmp_path)
+    _, model, s = _awq_artifact_dir(tmp, pinned=pinned)
+    meta, doc = artifacts.load_metadata(tmp), artifacts.read_norm_gain_doc(tmp)
+    if pinned:
+        # a gain trained further after the fold: the quotient would be wrong, the pinned file is not
+        import numpy as np
+        np.save(os.path.join(tmp, "norm_edits", "l0.npy"), np.zeros(H, dtype=np.float32))
+        doc["edits"]["model.layers.0.norm.weight"]["sha256"] = None
+    scales = artifacts.recover_awq_scales(model, tmp, meta, doc)
+    assert set(scales) == {"model.layers.0.mlp.gate_proj.weight", "model.layers.0.mlp.up_proj.weight"}
+    for got in scales.values():
+        assert got.dtype == torch.float32 and got.shape == (H,)
+        assert torch.allclose(got, s, rtol=(0 if pinned else 2e-6), atol=0)
+    # alpha == 0 entries contribute nothing; no document, no scales
+    assert artifacts.recover_awq_scales(model, tmp, meta, None) == {}
+    assert artifacts.recover_awq_scales(model, tmp, meta, {"edits": {}}) == {}
+
+
+def test_norm_edits_are_copied_into_the_model_once(tmp_path):
+    import numpy as np
+    tmp = str(tmp_path)
+    _, model, s = _awq_artifact_dir(tmp)
+    doc = artifacts.read_norm_gain_doc(tmp)
+    del doc["edits"]["model.layers.1.norm.weight"]                   # (its file is layer 0's: shape ok too)
+    before = model.model.layers[0].norm.weight.detach().clone()
+    applied = artifacts.apply_norm_gain_edits(model, tmp)
+    assert "model.layers.0.norm.weight" in applied
+    want = torch.from_numpy(np.load(os.path.join(tmp, "norm_edits", "l0.npy")))
+    assert torch.equal(model.model.layers[0].norm.weight.detach(), want)
+    assert torch.allclose((1 + before) / (1 + want), s, rtol=1e-5)
+    artifacts.apply_norm_gain_edits(model, tmp)                       # idempotent
+    assert torch.equal(model.model.layers[0].norm.weight.detach(), want)
+    assert artifacts.apply_norm_gain_edits(_LM(), str(tmp_path / "nothing_here")) == {}
+
+
+def test_awq_recovery_refusals(tmp_path):
+    import numpy as np
+    tmp = str(tmp_path)
+    # the legacy w/s fold: 1 + w' negative -> refused, not served approximately
+    _, model, _ = _awq_artifact_dir(tmp, legacy=True)
+    with pytest.raises(ValueError, match="zero-centred"):
+        artifacts.recover_awq_scales(model, tmp, artifacts.load_metadata(tmp), artifacts.read_norm_gain_doc(tmp))
+    # the tensors' own statistics disagree with the recovered scale
+    _, model, _ = _awq_artifact_dir(tmp, stats_off=True)
+    with pytest.raises(ValueError, match="s_min"):
+        artifacts.recover_awq_scales(model, tmp, artifacts.load_metadata(tmp), artifacts.read_norm_gain_doc(tmp))
+    _, model, s = _awq_artifact_dir(tmp)
+    meta, doc = artifacts.load_metadata(tmp), artifacts.read_norm_gain_doc(tmp)
+    # scales beyond (0, 1]: a model whose gain is not the one the edit was made from
+    other = _LM()
+    with torch.no_grad():
+        other.model.layers[0].norm.weight.fill_(3.0)
+    with pytest.raises(ValueError, match=r"\(0, 1\]"):
+        artifacts.recover_awq_scales(other, tmp, meta, doc)
+    # a parameter the model does not have; a corrupted edit file; a wrong shape
+    doc2 = {"edits": {"model.layers.9.norm.weight": doc["edits"]["model.layers.0.norm.weight"]}}
+    with pytest.raises(KeyError):
+        artifacts.recover_awq_scales(model, tmp, meta, doc2)
+    with open(os.path.join(tmp, "norm_gain_edits.json"), "w") as f:
+        json.dump(doc2, f)
+    with pytest.raises(KeyError):
+        artifacts.apply_norm_gain_edits(model, tmp, strict=True)
+    assert artifacts.apply_norm_gain_edits(model, tmp, strict=False) == {}
+    np.save(os.path.join(tmp, "norm_edits", "l0.npy"), np.zeros(H, dtype=np.float32))
+    with pytest.raises(ValueError, match="SHA256"):
+        artifacts.recover_awq_scales(model, tmp, meta, doc)
+    np.save(os.path.join(tmp, "norm_edits", "l0.npy"), np.zeros(H + 1, dtype=np.float32))
+    with pytest.raises(ValueError, match="shape"):
+        artifacts.recover_awq_scales(model, tmp, meta, doc, verify_sha=False)
+
+
+@torch.no_grad()
+def test_load_quant_model_recovers_and_applies_by_itself(tmp_path):
+    """load_quant_model on an AWQ set: the scales come from the edits (recovered on the pristine
+    gains), the gains are edited, and the rotated consumers carry the compensation: the same
+    module values as when the caller hands the scale map over."""
+    tmp = str(tmp_path)
+    _, model, s = _awq_artifact_dir(tmp)
+    state = {k: v.clone() for k, v in model.state_dict().items()}
+    auto, _ = loader.load_quant_model(tmp, "tiny", "cpu", forward="reference", dtype=torch.float32,
+                                      model=model)
+    gate = auto.model.layers[0].mlp.gate_proj
+    assert gate.awq_scale is not None and torch.allclose(gate.awq_scale.float(), s, rtol=2e-6)
+    assert gate._compensated() and auto.model.layers[1].mlp.gate_proj.awq_scale is None
+    edited = auto.model.layers[0].norm.weight
+    assert torch.allclose((1 + state["model.layers.0.norm.weight"]) / (1 + edited), s, rtol=1e-5)
+    # the caller's own map takes the recovered one's place; awq_compensation=False drops both
+    manual = _LM()
+    manual.load_state_dict(state)
+    names = ["model.layers.0.mlp.gate_proj.weight", "model.layers.0.mlp.up_proj.weight"]
+    manual, _ = loader.load_quant_model(tmp, "tiny", "cpu", forward="reference", dtype=torch.float32,
+                                        model=manual, awq_scales={n: s for n in names})
+    ids = torch.tensor([[3, 200, 77]])
+    assert rel_l2(auto(ids), manual(ids)) <= 1e-5        # the recovered scale is s to a few ulps
+    plain = _LM()
+    plain.load_state_dict(state)
+    plain, _ = loader.load_quant_model(tmp, "tiny", "cpu", forward="reference", dtype=torch.float32,
+                                       model=plain, awq_compensation=False)
+    assert plain.model.layers[0].mlp.gate_proj.awq_scale is None
+    assert rel_l2(plain(ids), auto(ids)) > 1e-3
+    # apply_norm_edits=False leaves the model's gains alone and recovers nothing
+    raw = _LM()
+    raw.load_state_dict(state)
+    raw, _ = loader.load_quant_model(tmp, "tiny", "cpu", forward="reference", dtype=torch.float32,
+                                     model=raw, apply_norm_edits=False)
+    assert torch.equal(raw.model.layers[0].norm.weight, state["model.layers.0.norm.weight"])
+    assert raw.model.layers[0].mlp.gate_proj.awq_scale is None
+
+
+@pytest.mark.gpu
+@torch.no_grad()
+def test_kernel_mode_matches_reference_mode_with_awq_compensation(tmp_path):
+    tmp = str(tmp_path)
+    _, model, s = _awq_artifact_dir(tmp)
+    state = {k: v.clone() for k, v in model.state_dict().items()}
+    ref_model, _ = loader.load_quant_model(tmp, "tiny", "cpu", forward="reference",
+                                           dtype=torch.float32, model=model)
+    base = _LM()
+    base.load_state_dict(state)
+    ker_model, _ = loader.load_quant_model(tmp, "tiny", "cuda:0", forward="kernel",
+                                           dtype=torch.float16, model=base)
+    assert ker_model.model.layers[0].mlp.gate_proj.awq_scale is not None
+    for ids in (torch.tensor([[17]]), torch.randint(0, V, (2, 9))):   # decode routes, prefill routes
+        y = ker_model(ids.to("cuda:0")).float().cpu()
+        assert rel_l2(y, ref_model(ids)) <= 2e-3
