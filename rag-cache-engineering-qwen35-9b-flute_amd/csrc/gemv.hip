@@ -414,8 +414,29 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         case 3: return launch_typed<BF16, 3>(plan, stream);
         case 2: return launch_typed<BF16, 2>(plan, stream);
         case 1: return launch_typed<BF16, 1>(plan, stream);
-        default: return launch_typed<BF16, 0>(plan, stream);
+        default: break;
     }
+    // mixed widths: the pairs deployed artifacts hold ((1,4) x45, (4,1) x24, (2,3) x3, (2,4) x6
+    // in upstream's census, flute_extended/__init__.py:226-233) have instantiations of their own
+    int b1 = plan.p.seg[0].st[0].bits, b2 = 0;
+    bool pair = true;
+    for (int i = 0; i < plan.p.nsegs; ++i) {
+        pair &= plan.p.seg[i].st[0].bits == b1;
+        if (plan.p.seg[i].nstreams == 2) {
+            if (b2 == 0) b2 = plan.p.seg[i].st[1].bits;
+            pair &= plan.p.seg[i].st[1].bits == b2;
+        }
+    }
+    if (pair) {
+        switch (10 * b1 + b2) {
+            case 14: return launch_typed<BF16, 14>(plan, stream);
+            case 41: return launch_typed<BF16, 41>(plan, stream);
+            case 23: return launch_typed<BF16, 23>(plan, stream);
+            case 24: return launch_typed<BF16, 24>(plan, stream);
+            default: break;
+        }
+    }
+    return launch_typed<BF16, 0>(plan, stream);
 }
 
 // Scratch memory a launch needs beyond its operands: partial sums of a K split, tickets,

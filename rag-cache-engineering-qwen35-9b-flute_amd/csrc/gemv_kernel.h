@@ -858,13 +858,20 @@ __device__ void run_stream(const GemvParams &p, const GemvSeg &sg, const GemvStr
     __syncthreads();
 }
 
-// BFIX != 0: every stream of the launch has this width (the common case, one
-// lean instantiation per width); BFIX == 0: widths are mixed and chosen per stream.
+// BFIX = 1..4: every stream of the launch has this width (the common case, one
+// instantiation per width); BFIX = 10 * b1 + b2: every weight's first stream is b1 bits wide
+// and its second one, where it has one, b2 (the mixed pairs of deployed artifacts: the code of
+// two widths only, which keeps the kernel in the register budget of three wavefronts per SIMD);
+// BFIX == 0: any mix, chosen per stream at run time (all four widths inlined: it spills).
 template <bool BF16, int BFIX>
 __device__ __forceinline__ void run_stream_any(const GemvParams &p, const GemvSeg &sg,
                                                const GemvStream &st, const LaneGeom &gm,
-                                               uint8_t *lds, float (&acc)[8]) {
-    if constexpr (BFIX != 0) {
+                                               uint8_t *lds, float (&acc)[8], int si) {
+    if constexpr (BFIX >= 10) {
+        if (si == 0) run_stream<BFIX / 10, BF16>(p, sg, st, gm, lds, acc);
+        else run_stream<BFIX % 10, BF16>(p, sg, st, gm, lds, acc);
+        return;
+    } else if constexpr (BFIX != 0) {
         run_stream<BFIX, BF16>(p, sg, st, gm, lds, acc);
         return;
     }
@@ -932,7 +939,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     // waits only for what was issued before it.  A rotated input is staged first: the
     // rotation needs most of the register file, and index loads held across it would
     // be spilled (and waited for) on the spot.
-    constexpr int BF = BFIX != 0 ? BFIX : 4;
+    constexpr int BF = BFIX >= 10 ? BFIX / 10 : (BFIX != 0 ? BFIX : 4);   // width of a first stream
     constexpr int XV = 2;                           // 16-byte activation loads per thread
     StreamRegs<BF> first;
     const uint16_t *x0 = sg.xsrc ? sg.xsrc : p.x;
@@ -989,7 +996,7 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
                     __syncthreads();
                 }
             } else {
-                run_stream_any<BF16, BFIX>(p, og, st, gm, lds, acc);
+                run_stream_any<BF16, BFIX>(p, og, st, gm, lds, acc, si);
             }
         }
 
