@@ -20,6 +20,7 @@ int entry_bytes_log2(int bits) { return bits >= 3 ? 2 : (bits == 2 ? 3 : 4); }
 
 struct Plan {
     GemvParams p;
+    int pair;               // 10 * b1 + b2 when the widths are a pair the lean kernel serves with two tables, else 0
     size_t lds_bytes;
     int grid_x;
     int threads;
@@ -275,6 +276,27 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     p.act_bf16 = act_dtype == FLUTE_BF16;
     p.x = (const uint16_t *)x;
 
+    // Mixed widths (and 3 + 3 bits) in the lean kernel: both tables of a weight stand side by
+    // side (4^b entries of 128 bytes each).  Decided here because it sets the table region;
+    // the launcher may still send the launch to the general kernel, which needs less.
+    plan->pair = 0;
+    {
+        int b1 = segs[0].b1, b2 = 0;
+        bool ok = true;
+        for (int i = 0; i < count; ++i) {
+            ok &= segs[i].b1 == b1 && segs[i].group_size >= 128;
+            if (segs[i].b2 > 0) {
+                if (b2 == 0) b2 = segs[i].b2;
+                ok &= segs[i].b2 == b2;
+            }
+        }
+        const int code = 10 * b1 + b2;
+        if (ok && (code == 41 || code == 14 || code == 33)) {
+            plan->pair = code;
+            const size_t both = (((size_t)1 << (2 * b1)) + ((size_t)1 << (2 * b2))) * 128;
+            if (both > tab_bytes) tab_bytes = both;
+        }
+    }
     size_t region0 = tab_bytes > scratch ? tab_bytes : scratch;
     region0 = (region0 + 255) & ~(size_t)255;
     p.lds_x = (int)region0;
@@ -348,6 +370,41 @@ flute_status launch_fast4(Plan &plan, hipStream_t stream) {
     return launch_fast4_grid<LPGL, NW, PF, BF16, false>(plan, gx, stream);
 }
 
+// The lean kernel with two resident tables (mixed widths); no walking grid.  Eight wavefronts
+// come with 8- or 16-row slices only (choose_shape).
+template <int LPGL, int NW, int PF, bool BF16, int BA, int BB>
+flute_status launch_pair_grid(const Plan &plan, hipStream_t stream) {
+    static std::atomic<bool> attr_done{false};
+    if (!attr_done) {
+        FLUTE_HIP_CHECK(hipFuncSetAttribute((const void *)gemv4_kernel<LPGL, NW, PF, BF16, false, BA, BB>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            (int)kLdsPerCU));
+        attr_done = true;
+    }
+    dim3 grid(plan.grid_x, plan.p.split);
+    hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, PF, BF16, false, BA, BB>), grid, dim3(NW * 64),
+                       plan.lds_bytes, stream, plan.p);
+    FLUTE_HIP_CHECK(hipGetLastError());
+    return FLUTE_OK;
+}
+template <bool BF16, int BA, int BB>
+flute_status launch_pair(Plan &plan, int nw, int pf, hipStream_t stream) {
+    plan.p.slices = 0;
+    switch (nw * 100 + plan.p.lpg_log2 * 10 + pf) {
+        case 442: return launch_pair_grid<4, 4, 2, BF16, BA, BB>(plan, stream);
+        case 444: return launch_pair_grid<4, 4, 4, BF16, BA, BB>(plan, stream);
+        case 452: return launch_pair_grid<5, 4, 2, BF16, BA, BB>(plan, stream);
+        case 454: return launch_pair_grid<5, 4, 4, BF16, BA, BB>(plan, stream);
+        case 462: return launch_pair_grid<6, 4, 2, BF16, BA, BB>(plan, stream);
+        case 464: return launch_pair_grid<6, 4, 4, BF16, BA, BB>(plan, stream);
+        case 842: return launch_pair_grid<4, 8, 2, BF16, BA, BB>(plan, stream);
+        case 844: return launch_pair_grid<4, 8, 4, BF16, BA, BB>(plan, stream);
+        case 852: return launch_pair_grid<5, 8, 2, BF16, BA, BB>(plan, stream);
+        case 854: return launch_pair_grid<5, 8, 4, BF16, BA, BB>(plan, stream);
+        default: return FLUTE_ERR_UNSUPPORTED;       // (not reached: the caller checks the shape)
+    }
+}
+
 // Loads a lane keeps in flight in the lean kernel: 4 when that divides the loads of a
 // wavefront, else 2; 0 when the launch does not fit the kernel (the wavefronts would get
 // different or odd numbers of loads: two loads feed one matrix product).
@@ -407,6 +464,16 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
             case 4: return launch_fast4_shape<4, BF16>(plan, nw, stream);
             case 5: return launch_fast4_shape<5, BF16>(plan, nw, stream);
             default: return launch_fast4_shape<6, BF16>(plan, nw, stream);
+        }
+    }
+    if (plan.pair && one_group && one_input && es == 7 && luts_aligned &&
+        (nw == 4 || (nw == 8 && plan.p.lpg_log2 <= 5)) && pick_prefetch(plan, nw) != 0 &&
+        tuning().gemv_no_fast == 0) {
+        const int pf = pick_prefetch(plan, nw);
+        switch (plan.pair) {
+            case 41: return launch_pair<BF16, 4, 1>(plan, nw, pf, stream);
+            case 14: return launch_pair<BF16, 1, 4>(plan, nw, pf, stream);
+            default: return launch_pair<BF16, 3, 3>(plan, nw, pf, stream);
         }
     }
     switch (bits) {

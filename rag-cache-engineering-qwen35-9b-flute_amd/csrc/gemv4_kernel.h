@@ -48,6 +48,8 @@
 // a one-slice launch.
 #pragma once
 
+#include <type_traits>
+
 #include "gemv_kernel.h"
 
 namespace flute {
@@ -76,21 +78,44 @@ __device__ __forceinline__ float quad_lane(float v) {
         float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 
-// Sixteen index bytes, read once: non-temporal, so they do not displace the
-// activations and LUT rows that every workgroup shares from the caches.
-__device__ __forceinline__ uint4 load_idx16(const uint8_t *p) {
-    typedef const __attribute__((address_space(1))) gv_u4_t *GlobalQuad;       // global, not flat
-    const gv_u4_t v = __builtin_nontemporal_load((GlobalQuad)(uintptr_t)p);
-    return make_uint4(v.x, v.y, v.z, v.w);
+// Index bytes are read once: non-temporal loads, so they do not displace the activations
+// and LUT rows that every workgroup shares from the caches.
+// One quarter of a chunk of a B-bit stream: 16 pairs of codes, 4 * B bytes, read once.
+template <int B>
+struct IdxQuarter {
+    uint32_t d[B];
+};
+template <int B>
+__device__ __forceinline__ IdxQuarter<B> load_idx(const uint8_t *p) {
+    typedef uint32_t vec_t __attribute__((ext_vector_type(B == 3 ? 3 : B)));
+    typedef const __attribute__((address_space(1))) vec_t *GlobalVec;              // global, not flat
+    IdxQuarter<B> r;
+    if constexpr (B == 1) {
+        typedef const __attribute__((address_space(1))) uint32_t *GlobalWord;
+        r.d[0] = __builtin_nontemporal_load((GlobalWord)(uintptr_t)p);
+    } else {
+        const vec_t v = __builtin_nontemporal_load((GlobalVec)(uintptr_t)p);
+#pragma unroll
+        for (int i = 0; i < B; ++i) r.d[i] = v[i];
+    }
+    return r;
+}
+// The 2B-bit code of pair pp (0..15) of a quarter (all indices constant after unrolling).
+template <int B>
+__device__ __forceinline__ uint32_t quarter_code(const IdxQuarter<B> &q, int pp) {
+    const int bit = 2 * B * pp, dw = bit >> 5, sh = bit & 31;
+    if (sh + 2 * B <= 32) return __builtin_amdgcn_ubfe(q.d[dw], sh, 2 * B);
+    return __builtin_amdgcn_alignbit(q.d[dw + 1 < B ? dw + 1 : dw], q.d[dw], sh) & ((1u << (2 * B)) - 1u);
 }
 
-// One LUT row of sixteen 16-bit values through the scalar cache (the pointer is
-// wavefront-uniform and 4-byte aligned).
+// One LUT row of 2^B 16-bit values through the scalar cache (the pointer is
+// wavefront-uniform and 4-byte aligned); dwords beyond the row stay zero.
+template <int B = 4>
 __device__ __forceinline__ void load_lut_row(const uint16_t *lut, uint32_t (&d)[8]) {
     typedef const __attribute__((address_space(4))) uint32_t *ConstWord;
     ConstWord p = (ConstWord)(const void *)lut;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) d[i] = p[i];
+    for (int i = 0; i < 8; ++i) d[i] = i < (1 << B) / 2 ? p[i] : 0u;
 }
 
 // Value c (0..15) of a LUT row held as eight uniform dwords.
@@ -171,7 +196,12 @@ __device__ __forceinline__ void rotate_piece(uint4 &v, const float (&sg)[8], con
 // four-wavefront workgroups fit a CU.
 // WALK: the instantiation for resident grids that walk over the row slices (p.slices > 0);
 // launches of one workgroup per slice use the one without that control path.
-template <int LPGL, int NW, int PF, bool BF16, bool WALK = false>
+// BA, BB: widths of every weight's first stream and (where it has one) second stream.  (4, 4) is
+// the kernel described above: one table, rebuilt between the passes.  Any other pair (the mixed
+// pairs of deployed artifacts, (3, 3)) has small tables: both are built before an output's first
+// loop (the first at offset 0, the second behind it) and the two K loops run back to back, with
+// no barrier and no table build between them.
+template <int LPGL, int NW, int PF, bool BF16, bool WALK = false, int BA = 4, int BB = 4>
 __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int ES = 7;
@@ -190,6 +220,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     static_assert(NT >= 256, "one thread per table entry at least");
     static_assert(PF % 2 == 0 && PF >= PF0, "loads are consumed in pairs");
     static_assert(!WALK || NW == 4, "the alternating sum areas of a walking grid are sized for four wavefronts");
+    constexpr bool TWO = !(BA == 4 && BB == 4);     // two resident tables
+    static_assert(!TWO || !WALK, "walking grids: the (4, 4) kernel");
+    constexpr int TAB_A = (1 << (2 * BA)) * STRIDE; // bytes of the first table
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     warm_kernargs<(int)sizeof(GemvParams)>(kp);
@@ -238,10 +271,12 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     float *red = (float *)(lds + p.lds_red);        // [2][NW][4][8] partial row sums
 
     // lane-constant pieces of the addresses
-    const uint32_t unit_bytes = GPI * 4096u;
-    const uint32_t lane0 = (uint32_t)gsub * 4096u + (uint32_t)cgl * 256u +
-                           (uint32_t)kg * 64u + (uint32_t)kt * 16u + (uint32_t)w * unit_bytes;
-    constexpr uint32_t step = NW * GPI * 4096u;
+    // (a B-bit stream: tiles of 1024 * B bytes, chunk groups of 64 * B, chunks of 16 * B,
+    // quarters of 4 * B)
+    const uint32_t lane_unit = (uint32_t)gsub * 1024u + (uint32_t)cgl * 64u + (uint32_t)kg * 16u +
+                               (uint32_t)kt * 4u + (uint32_t)w * (GPI * 1024u);
+    const uint32_t lane0 = lane_unit * BA, lane0B = lane_unit * BB;
+    constexpr uint32_t step = NW * GPI * 1024u * BA, stepB = NW * GPI * 1024u * BB;
     // Lookup addresses are formed as absolute LDS addresses, so the (zero) base of
     // the dynamic LDS block is folded into the per-lane replica offset once.
     typedef const __attribute__((address_space(3))) uint32_t *LdsWord;
@@ -251,6 +286,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // address of byte 0 be formed as shift + and-or, two instructions like the other bytes.
     __builtin_assume(lds_base == 0);
     const uint32_t slot = lds_base + (uint32_t)(L & 31) * 4u;
+    const uint32_t slotB = slot + (TWO ? TAB_A : 0);
     const int e_own = tid & 255;                    // table entry this thread writes
     const int share = tid >> 8;
 
@@ -265,18 +301,19 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         const GemvStream st = kp->seg[sg].st[si_];
         const int t = sl_ / SPT, cg0 = (sl_ % SPT) * (RW >> 3);
         const int grp = min((t * 128) >> __builtin_ctz(kp->seg[sg].gs), kp->seg[sg].lut_rows - 1);
-        qr = st.q + ((size_t)t * G + g_lo) * 4096u + (uint32_t)cg0 * 256u;
-        lutp = st.lut + ((size_t)grp << 4);
+        const int B = si_ ? BB : BA;
+        qr = st.q + ((size_t)t * G + g_lo) * (1024u * B) + (uint32_t)cg0 * (64u * B);
+        lutp = st.lut + ((size_t)grp << B);
     };
     // Index loads are addressed as (uniform base + unit offset) in scalar registers
     // plus one lane-constant 32-bit offset, so no per-load address lives in vector
     // registers; every load is unconditional, so the compiler knows how many are in
     // flight at each point and waits for exactly the ones a product needs.
-    auto first_units = [&](const uint8_t *qr, uint4 (&qq)[PF], int from) {
+    auto first_units = [&](const uint8_t *qr, IdxQuarter<BA> (&qq)[PF], int from) {
 #pragma unroll
         for (int n = 0; n < PF; ++n) {
             if (n >= from) {
-                qq[n] = load_idx16(qr + (size_t)n * step + lane0);
+                qq[n] = load_idx<BA>(qr + (size_t)n * step + lane0);
                 __builtin_amdgcn_sched_barrier(0);  // issue order = consumption order
             }
         }
@@ -291,6 +328,38 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         uint8_t *ent = lds + e_own * STRIDE + share * (CPT * 16);
 #pragma unroll
         for (int k = 0; k < CPT; ++k) *(uint4 *)(ent + (((k + tid) & (CPT - 1)) << 4)) = v4;
+    };
+    // A table of a narrower stream (4^B entries, at most 64): one thread per entry writes all
+    // the replicas of its entry.
+    auto write_small_table = [&](const uint32_t (&row)[8], auto width, uint32_t base) {
+        constexpr int B = decltype(width)::value;
+        if (tid < (1 << (2 * B))) {
+            const uint32_t v = lut_value(row, tid & ((1 << B) - 1)) | (lut_value(row, tid >> B) << 16);
+            const uint4 v4 = make_uint4(v, v, v, v);
+            uint8_t *ent = lds + base + tid * STRIDE;
+#pragma unroll
+            for (int k = 0; k < CHUNKS; ++k) *(uint4 *)(ent + (((k + tid) & (CHUNKS - 1)) << 4)) = v4;
+        }
+    };
+    // the tables of one output: the first stream's, and (two resident tables) the second's
+    auto write_tables = [&](const uint32_t (&rowA)[8], const uint32_t (&rowB)[8], bool second) {
+        if constexpr (BA == 4) write_table(rowA);
+        else write_small_table(rowA, std::integral_constant<int, BA>(), 0u);
+        if constexpr (TWO) {
+            if (second) {
+                if constexpr (BB == 4) {
+                    // (a 4-bit second stream behind a narrow first one: the full-size writer at the
+                    // second table's base)
+                    const uint32_t v = lut_value(rowB, e_own & 15) | (lut_value(rowB, e_own >> 4) << 16);
+                    const uint4 v4 = make_uint4(v, v, v, v);
+                    uint8_t *ent = lds + TAB_A + e_own * STRIDE + share * (CPT * 16);
+#pragma unroll
+                    for (int k = 0; k < CPT; ++k) *(uint4 *)(ent + (((k + tid) & (CPT - 1)) << 4)) = v4;
+                } else {
+                    write_small_table(rowB, std::integral_constant<int, BB>(), (uint32_t)TAB_A);
+                }
+            }
+        }
     };
 
     // Activations in operand order: for load unit u (GPI tiles) the 8 bytes
@@ -316,12 +385,23 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const uint8_t *qrow;
     const uint16_t *lut;
     pass_ptrs(sl, 0, 0, qrow, lut);
-    uint32_t lrow[8];
-    load_lut_row(lut, lrow);
+    uint32_t lrow[8], lrowB[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+    load_lut_row<BA>(lut, lrow);
+    bool second0 = false;                           // two tables: this output has a second stream
+    if constexpr (TWO) {
+        second0 = kp->seg[si0].nstreams == 2;
+        if (second0) {
+            const uint8_t *q_unused;
+            const uint16_t *lutB;
+            pass_ptrs(sl, 0, 1, q_unused, lutB);
+            load_lut_row<BB>(lutB, lrowB);
+        }
+    }
     const uint16_t *staged_x = kp->seg[si0].xsrc ? kp->seg[si0].xsrc : p.x;
     const float *staged_signs = kp->seg[si0].signs, *staged_awq = kp->seg[si0].awq;
     const bool x_plain = staged_signs == nullptr;   // plain copy
-    uint4 q[PF];
+    IdxQuarter<BA> q[PF];
+    IdxQuarter<BB> q2[PF];
     // bfloat16 activations in front of a float16 LUT: the staged units hold x * 2^-xshift,
     // xshift chosen per wavefront (per workgroup when the input is rotated)
     const bool convert = !BF16 && p.act_bf16;       // uniform
@@ -369,10 +449,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int n = 0; n < PF0; ++n) {
-            q[n] = load_idx16(qrow + (size_t)n * step + lane0);
+            q[n] = load_idx<BA>(qrow + (size_t)n * step + lane0);
             __builtin_amdgcn_sched_barrier(0);
         }
-        write_table(lrow);
+        write_tables(lrow, lrowB, second0);
         first_units(qrow, q, PF0);
         if (rot_inwave) {
             const int nst = 31 - __builtin_clz((unsigned)p.fht_block);
@@ -430,7 +510,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 stage8(j, !convert ? v : finite ? bf16_to_f16_top8(v, adj) : bf16_to_f16_scaled8(v, 0));
             }
         }
-        write_table(lrow);
+        write_tables(lrow, lrowB, second0);
         __builtin_amdgcn_sched_barrier(0);
         first_units(qrow, q, 0);
     } else {
@@ -438,11 +518,11 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         // index loads travel while it runs.
 #pragma unroll
         for (int n = 0; n < PF0; ++n) {
-            q[n] = load_idx16(qrow + (size_t)n * step + lane0);
+            q[n] = load_idx<BA>(qrow + (size_t)n * step + lane0);
             __builtin_amdgcn_sched_barrier(0);
         }
         xshift = stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
-        write_table(lrow);
+        write_tables(lrow, lrowB, second0);
         __builtin_amdgcn_sched_barrier(0);
         first_units(qrow, q, PF0);
     }
@@ -496,8 +576,135 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         kp->seg[si0].out[n] = round_act(y, p.act_bf16);
     };
 
-    bool same_table = false;                        // walking: the next slice reuses the table
+    // ---- K loop pieces, generic in the width of the stream ----------------------------------
+    // One step = two units (two loads of this lane) = 32 lookups and 8 matrix products.
+    auto operand_b = [&](int m0, int m1) -> gv_u4_t {
+        const int u0 = w + m0 * NW, u1 = w + m1 * NW;
+        if (x_direct) {
+            const uint2 xa = xs64[u0 * (16 * GPI) + xoff], xb = xs64[u1 * (16 * GPI) + xoff];
+            return (gv_u4_t){xa.x, xa.y, xb.x, xb.y};
+        }
+        const int a0 = u0 * (32 * GPI) + xnat, a1 = u1 * (32 * GPI) + xnat;
+        return (gv_u4_t){xs32[a0], xs32[a0 + 4], xs32[a1], xs32[a1 + 4]};
+    };
+    // per row group v, eight lookups feed two matrix products; pair pp = v * 4 + d * 2 + s2 of a
+    // quarter, an operand is (s2 = 0, 1) of both units
+    auto unit_pair = [&](const auto &qa, const auto &qb, gv_u4_t Bop, uint32_t tslot, auto width) {
+        constexpr int B = decltype(width)::value;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            auto look = [&](const IdxQuarter<B> &qq, int j) -> uint32_t {
+                if constexpr (B == 4 && !TWO) {
+                    // a whole byte of dword v; byte 0: shift, then one and-or (the slot lies
+                    // below the stride, the table at offset 0)
+                    const uint32_t wq = qq.d[v];
+                    if (j == 0) return *(LdsWord)(((wq << ES) & (0xffu << ES)) | tslot);
+                    return *(LdsWord)((((wq >> (8 * j)) & 0xffu) << ES) + tslot);
+                } else {
+                    return *(LdsWord)((quarter_code<B>(qq, v * 4 + j) << ES) + tslot);
+                }
+            };
+            const gv_u4_t A0 = {look(qa, 0), look(qa, 1), look(qb, 0), look(qb, 1)};
+            const gv_u4_t A1 = {look(qa, 2), look(qa, 3), look(qb, 2), look(qb, 3)};
+            acc[v * 2] = gv_mfma<BF16>(A0, Bop, acc[v * 2]);
+            acc[v * 2 + 1] = gv_mfma<BF16>(A1, Bop, acc[v * 2 + 1]);
+        }
+    };
+    // The K range of one stream of width B held in qc, refilled from qcur; the last group's
+    // registers are refilled with the first loads of what follows: a stream of width BN from
+    // qnext into qn (nothing when last).
+    auto k_loop = [&](auto &qc, const uint8_t *qcur, uint32_t lane_c, uint32_t step_c, uint32_t tslot,
+                      auto width, auto &qn, const uint8_t *qnext, uint32_t lane_n, uint32_t step_n,
+                      auto width_next, bool has_next) {
+        constexpr int B = decltype(width)::value, BN = decltype(width_next)::value;
+        int nb = 0;
+        __builtin_amdgcn_s_setprio(2);
+        for (; nb + 2 * PF <= my_units; nb += PF) {          // every refill exists
+#pragma unroll
+            for (int n = 0; n < PF; n += 2) {
+                const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
+                unit_pair(qc[n], qc[n + 1], Bop, tslot, width);
+                __builtin_amdgcn_sched_barrier(0);
+                qc[n] = load_idx<B>(qcur + (size_t)(nb + n + PF) * step_c + lane_c);
+                qc[n + 1] = load_idx<B>(qcur + (size_t)(nb + n + 1 + PF) * step_c + lane_c);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if (!has_next) __builtin_amdgcn_s_setprio(1);
+        if (has_next) {
+#pragma unroll
+            for (int n = 0; n < PF; n += 2) {
+                const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
+                unit_pair(qc[n], qc[n + 1], Bop, tslot, width);
+                __builtin_amdgcn_sched_barrier(0);
+                qn[n] = load_idx<BN>(qnext + (size_t)n * step_n + lane_n);
+                qn[n + 1] = load_idx<BN>(qnext + (size_t)(n + 1) * step_n + lane_n);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int n = 0; n < PF; n += 2) {
+                const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
+                unit_pair(qc[n], qc[n + 1], Bop, tslot, width);
+            }
+        }
+        if (!has_next) __builtin_amdgcn_s_setprio(0);
+    };
+    // ---- end of an output: D[i][j] with i = (rb, kt) in (lane >> 4, register) and
+    //      j = (rb', kt') in lane & 15.  The lanes with rb' == rb keep register kt';
+    //      a quad sum folds kt'; the activation scaling is undone here (exact). -----
+    auto end_of_output = [&](int so_, int par_) {
+        const bool keep = rb == kg;                 // here L >> 4 is the matrix row block
+#pragma unroll
+        for (int a = 0; a < 8; ++a) {
+            // lane kt' of a quad holds the wanted term in register kt': each register is
+            // read from its own lane of the quad, summed as (0 + 1) + (2 + 3)
+            const float v = (quad_lane<0x00>(acc[a][0]) + quad_lane<0x55>(acc[a][1])) +
+                            (quad_lane<0xAA>(acc[a][2]) + quad_lane<0xFF>(acc[a][3]));
+            if (keep && kt == 0)
+                red[par_ * (2 * NW * 32) + (so_ * NW + w) * 32 + rb * 8 + a] = ldexpf(v, xshift);
+            acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    };
+    const auto WA = std::integral_constant<int, BA>();
+    const auto WB = std::integral_constant<int, BB>();
+
     int par = 0;                                    // walking: the partial sums alternate between two areas
+    if constexpr (TWO) {
+        // ---- two resident tables: per output, [both tables] barrier, loop A, loop B ----------
+        for (so = 0; so < nout; ++so) {
+            const int sg = so == 1 ? 1 : si0;
+            const bool second = kp->seg[sg].nstreams == 2;
+            if (so > 0) write_tables(lrow, lrowB, second);  // (the first output's: in the prologue)
+            // the LUT rows of the next output travel under this output's loops
+            const bool more = so + 1 < nout;
+            const uint8_t *qa_next = qrow, *qb_cur = qrow, *q_unused;
+            const uint16_t *lutn;
+            bool second_next = false;
+            if (second) pass_ptrs(sl, so, 1, qb_cur, lutn);
+            if (more) {
+                second_next = kp->seg[1].nstreams == 2;
+                pass_ptrs(sl, so + 1, 0, qa_next, lutn);
+                load_lut_row<BA>(lutn, lrow);
+                if (second_next) {
+                    pass_ptrs(sl, so + 1, 1, q_unused, lutn);
+                    load_lut_row<BB>(lutn, lrowB);
+                }
+            }
+            __syncthreads();                        // publishes the tables (and the staged activations)
+            if (second) {
+                k_loop(q, qrow, lane0, step, slot, WA, q2, qb_cur, lane0B, stepB, WB, true);
+                k_loop(q2, qb_cur, lane0B, stepB, slotB, WB, q, qa_next, lane0, step, WA, more);
+            } else {
+                k_loop(q, qrow, lane0, step, slot, WA, q, qa_next, lane0, step, WA, more);
+            }
+            end_of_output(so, 0);
+            if (!more) break;
+            __syncthreads();                        // the table region is rewritten next
+            qrow = qa_next;
+        }
+    } else {
+    bool same_table = false;                        // walking: the next slice reuses the table
     for (bool first = true;; first = false) {
         const int sg = so == 1 ? 1 : si0;
         if (!first && !same_table) {
@@ -535,85 +742,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         // publishes the table; with the table kept, the alternating sum areas make it unnecessary
         if (!same_table) __syncthreads();
 
-        // ---- K loop -----------------------------------------------------------------
-        // One step = two 16-byte loads of this lane = 32 lookups and 8 matrix products.
-        auto operand_b = [&](int m0, int m1) -> gv_u4_t {
-            const int u0 = w + m0 * NW, u1 = w + m1 * NW;
-            if (x_direct) {
-                const uint2 xa = xs64[u0 * (16 * GPI) + xoff], xb = xs64[u1 * (16 * GPI) + xoff];
-                return (gv_u4_t){xa.x, xa.y, xb.x, xb.y};
-            }
-            const int a0 = u0 * (32 * GPI) + xnat, a1 = u1 * (32 * GPI) + xnat;
-            return (gv_u4_t){xs32[a0], xs32[a0 + 4], xs32[a1], xs32[a1 + 4]};
-        };
-        // two units (two 16-byte loads of this lane): per row group v, eight lookups feed two
-        // matrix products
-        auto unit_pair = [&](const uint4 &qa, const uint4 &qb, gv_u4_t B) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const uint32_t wa = v == 0 ? qa.x : v == 1 ? qa.y : v == 2 ? qa.z : qa.w;
-                const uint32_t wb = v == 0 ? qb.x : v == 1 ? qb.y : v == 2 ? qb.z : qb.w;
-                // byte j of a dword: d = j >> 1, s2 = j & 1; an operand is (s2 = 0, 1) of both units
-                auto look = [&](uint32_t wq, int j) -> uint32_t {
-                    // byte 0: shift, then one and-or (the slot lies below the stride)
-                    if (j == 0) return *(LdsWord)(((wq << ES) & (0xffu << ES)) | slot);
-                    return *(LdsWord)((((wq >> (8 * j)) & 0xffu) << ES) + slot);
-                };
-                const gv_u4_t A0 = {look(wa, 0), look(wa, 1), look(wb, 0), look(wb, 1)};
-                const gv_u4_t A1 = {look(wa, 2), look(wa, 3), look(wb, 2), look(wb, 3)};
-                acc[v * 2] = gv_mfma<BF16>(A0, B, acc[v * 2]);
-                acc[v * 2 + 1] = gv_mfma<BF16>(A1, B, acc[v * 2 + 1]);
-            }
-        };
-        int nb = 0;
-        __builtin_amdgcn_s_setprio(2);
-        for (; nb + 2 * PF <= my_units; nb += PF) {          // every refill exists
-#pragma unroll
-            for (int n = 0; n < PF; n += 2) {
-                const gv_u4_t B = operand_b(nb + n, nb + n + 1);
-                unit_pair(q[n], q[n + 1], B);
-                __builtin_amdgcn_sched_barrier(0);
-                q[n] = load_idx16(qrow + (size_t)(nb + n + PF) * step + lane0);
-                q[n + 1] = load_idx16(qrow + (size_t)(nb + n + 1 + PF) * step + lane0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        if (!has_next) __builtin_amdgcn_s_setprio(1);
-        if (has_next) {
-#pragma unroll
-            for (int n = 0; n < PF; n += 2) {
-                const gv_u4_t B = operand_b(nb + n, nb + n + 1);
-                unit_pair(q[n], q[n + 1], B);
-                __builtin_amdgcn_sched_barrier(0);
-                q[n] = load_idx16(qnext + (size_t)n * step + lane0);
-                q[n + 1] = load_idx16(qnext + (size_t)(n + 1) * step + lane0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
-#pragma unroll
-            for (int n = 0; n < PF; n += 2) {
-                const gv_u4_t B = operand_b(nb + n, nb + n + 1);
-                unit_pair(q[n], q[n + 1], B);
-            }
-        }
+        k_loop(q, qrow, lane0, step, slot, WA, q, qnext, lane0, step, WA, has_next);
 
-        if (!has_next) __builtin_amdgcn_s_setprio(0);
-        // ---- end of an output: D[i][j] with i = (rb, kt) in (lane >> 4, register) and
-        //      j = (rb', kt') in lane & 15.  The lanes with rb' == rb keep register kt';
-        //      a quad sum folds kt'; the activation scaling is undone here (exact). -----
-        if (out_ends) {
-            const bool keep = rb == kg;             // here L >> 4 is the matrix row block
-#pragma unroll
-            for (int a = 0; a < 8; ++a) {
-                // lane kt' of a quad holds the wanted term in register kt': each register is
-                // read from its own lane of the quad, summed as (0 + 1) + (2 + 3)
-                const float v = (quad_lane<0x00>(acc[a][0]) + quad_lane<0x55>(acc[a][1])) +
-                                (quad_lane<0xAA>(acc[a][2]) + quad_lane<0xFF>(acc[a][3]));
-                if (keep && kt == 0)
-                    red[par * (2 * NW * 32) + (so * NW + w) * 32 + rb * 8 + a] = ldexpf(v, xshift);
-                acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-            }
-        }
+        if (out_ends) end_of_output(so, par);
         if (!has_next) break;
         __syncthreads();                            // the table region is rewritten next
         if (slice_ends) {
@@ -632,6 +763,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         si = nsi;
         qrow = qnext;
         lut = lutn;
+    }
     }
     __syncthreads();
 

@@ -15,7 +15,9 @@ import torch
 import flute_extended as fx
 import flute_oracle as O
 from _util import make_weight, make_x, rel_l2
-from flute_extended import _C
+import ctypes
+
+from flute_extended import _C, _lib
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -478,3 +480,118 @@ def test_compiled_binding_gives_the_python_binding_s_outputs():
     _C.native.qgemm_gemv_mlp(x, table(outs[0], outs[1]), outs[5])
     torch.cuda.synchronize()
     assert torch.equal(outs[4], outs[5]) and outs[4].abs().sum() > 0
+
+
+# ---- the width pairs of deployed artifacts in the lean kernel: two resident tables ------------
+# (upstream's census of two-stream layers: (1,4) x45, (4,1) x24, (3,3) x61,
+#  flute_extended/__init__.py:226-233; its kernel: include/flute/gemv.cuh:187-288)
+
+def _lib_desc(w, signs=None, block=0):
+    """flute_linear of a test weight (device tensors), for calls straight through the C ABI."""
+    d = _lib.FluteLinear()
+    d.q1, d.lut1, d.q1_bytes = w["blob_d"].data_ptr(), w["lut_d"].data_ptr(), w["blob_d"].numel()
+    if w["bits2"]:
+        d.q2, d.lut2, d.q2_bytes = w["blob2_d"].data_ptr(), w["lut2_d"].data_ptr(), w["blob2_d"].numel()
+    d.N, d.K, d.b1, d.b2, d.group_size = w["N"], w["K"], w["bits"], w["bits2"], w["gs"]
+    d.lut_rows = w["lut"].shape[0]
+    d.lut_dtype = _lib.F16 if w["lut"].dtype == torch.float16 else _lib.BF16
+    if signs is not None:
+        w["_signs_keep"] = signs
+        d.signs, d.rot_block = signs.data_ptr(), block
+    return d
+
+
+PAIR_SHAPES = [
+    # N, K: which launch shape the library picks (rows per workgroup / wavefronts / loads in flight)
+    (512, 1024),      # 8 rows, 4 wavefronts, 2 loads
+    (2048, 4096),     # 8 rows, 4 wavefronts, 4 loads
+    (4096, 12288),    # 16 rows, 8 wavefronts
+    (12288, 4096),    # 16 rows, 4 wavefronts: the MLP up-projection
+    (16384, 2048),    # 32 rows
+]
+
+
+@pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3)])
+@pytest.mark.parametrize("N,K", PAIR_SHAPES)
+def test_width_pairs_two_resident_tables(N, K, bits, bits2, act):
+    """Every row against the fp64 oracle at the reference forward's rounding point, repeats bit
+    identical, and the same weight through the general kernel (FLUTE_GEMV_NO_FAST) within the
+    same tolerance of it."""
+    w = make_weight(N, K, bits, 128, seed=N + K + 10 * bits + bits2, bits2=bits2, act_dtype=act,
+                    device=DEV)
+    x = make_x(1, K, seed=17, dtype=act)
+    y = _run(w, x).cpu()
+    assert y.dtype == act
+    assert rel_l2(y, _exact(w, x).to(act)) <= TOL
+    assert torch.equal(y, _run(w, x).cpu())
+
+
+@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3)])
+def test_width_pairs_one_hot_rows_are_the_sum_of_both_dequantised_columns(bits, bits2):
+    """x = e_k: the output is W1[:, k] + W2[:, k], one fp32 add of two 16-bit values rounded once:
+    bit-exact against the dequantised columns for k in every quarter of a tile."""
+    N, K = 512, 1024
+    w = make_weight(N, K, bits, 128, seed=5, bits2=bits2, device=DEV)
+    W1 = O.dequant(w["blob"].numpy(), w["lut"], N, K, 128, bits)
+    W2 = O.dequant(w["blob2"].numpy(), w["lut2"], N, K, 128, bits2)
+    for k in (0, 17, 63, 64, 511, 1000):
+        x = torch.zeros(1, K, dtype=torch.float16)
+        x[0, k] = 1.0
+        y = _run(w, x).cpu()
+        assert torch.equal(y[0], (W1[:, k].float() + W2[:, k].float()).half())
+
+
+@pytest.mark.parametrize("split", [2, 4])
+@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3)])
+def test_width_pairs_with_a_k_split_residual_and_bias(bits, bits2, split):
+    w = make_weight(1024, 4096, bits, 128, seed=9, bits2=bits2, rank=8, bias=True, device=DEV)
+    x = make_x(1, 4096, seed=4)
+    y = _run(w, x, split=split).cpu()
+    assert rel_l2(y, _exact(w, x).half()) <= TOL
+    assert torch.equal(y, _run(w, x, split=split).cpu())
+
+
+@pytest.mark.parametrize("block", [0, 128])
+def test_width_pair_with_a_fused_rotation(block):
+    """(4, 1) behind the rotation in the prologue: the rotated row feeds both streams; equal
+    to rotating first and calling the unrotated launch, bit for bit."""
+    import fht
+    N, K = 1024, 4096
+    w = make_weight(N, K, 4, 128, seed=12, bits2=1, device=DEV)
+    x = make_x(1, K, seed=6)
+    signs = O.rotation_signs(K, 5)
+    d = _lib_desc(w, signs.to(DEV), block)
+    y = torch.zeros(1, N, dtype=torch.float16, device=DEV)
+    xd = x.to(DEV)
+    assert _lib.lib.flute_gemv(ctypes.byref(d), xd.data_ptr(), y.data_ptr(), _lib.F16, 0,
+                               torch.cuda.current_stream().cuda_stream) == 0, _lib.last_error()
+    xr = torch.empty_like(xd)
+    assert _lib.lib.flute_fht(xd.data_ptr(), d.signs, None, xr.data_ptr(), 1, K, _lib.F16, 0, block,
+                              torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y.cpu(), _run(w, xr.cpu()).cpu())
+    ref = O.block_fht_reference(x, block, signs) if block else O.fht_reference(x, signs)
+    assert rel_l2(y.cpu(), _exact(w, ref).half()) <= TOL
+
+
+def test_merged_gate_up_with_two_stream_members():
+    """gate (4, 1) + up (4, 1), and gate (4, 1) + up (4, 0): tables of both streams are rebuilt
+    per output; SiLU * mul of the fp32 sums, one rounding."""
+    N, K = 2048, 4096
+    x = make_x(1, K, seed=3)
+    for up_bits2 in (1, 0):
+        g = make_weight(N, K, 4, 128, seed=21, bits2=1, device=DEV)
+        u = make_weight(N, K, 4, 128, seed=22, bits2=up_bits2, device=DEV)
+        out = torch.zeros(1, N, dtype=torch.float16, device=DEV)
+        row = lambda w_: [w_["blob_d"].data_ptr(), w_["lut_d"].data_ptr(),
+                          w_["blob2_d"].data_ptr() if w_["bits2"] else 0,
+                          w_["lut2_d"].data_ptr() if w_["bits2"] else 0, 0, 0, 0, 0, N, 0, 4, w_["bits2"],
+                          128, 0, 0]
+        table = torch.tensor([row(g), row(u)], dtype=torch.int64)
+        y = fx.qgemm_gemv_mlp(x.to(DEV), table, out).cpu()
+        ref = O.silu_mul_exact(_exact(g, x), _exact(u, x)).half()
+        assert rel_l2(y, ref) <= TOL
+        y1 = y.clone()
+        fx.qgemm_gemv_mlp(x.to(DEV), table, out)
+        assert torch.equal(out.cpu(), y1)
