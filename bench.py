@@ -236,6 +236,31 @@ class _Gemv:
         return res
 
 
+def _read_probe(torch, _lib, dev, keep):
+    """What one launch that only reads the 24 MiB of a weight's index blob reaches (same
+    rotation of cold blobs, same graph timing as the headline): the level the GEMV's launch can
+    be read against.  Grid size and loads in flight swept, best taken."""
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    nbytes = keep[0][0].numel()
+    best = None
+    for wgs in (768, 1536, 3072):
+        for pf in (4, 8):
+            def call(i, wgs=wgs, pf=pf):
+                st = _lib.lib.flute_read_probe(keep[i % len(keep)][0].data_ptr(), nbytes, wgs, pf,
+                                               sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+                if st != 0:
+                    raise RuntimeError(_lib.last_error())
+            n = max(96, len(keep))
+            us = _time_graph(torch, lambda: [call(i) for i in range(n)], reps=7) / n * 1e3
+            if best is None or us < best[0]:
+                best = (us, wgs, pf)
+    us, wgs, pf = best
+    return {"us_per_call": round(us, 3), "gbs": round(nbytes / us / 1e3, 1),
+            "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": nbytes,
+            "workgroups": wgs, "loads_in_flight": pf, "parity_rel_l2": 0.0,
+            "what": "flute_read_probe: 16-byte non-temporal loads only, no table, no arithmetic"}
+
+
 def _copy_desc(_lib, ctypes, d):
     c = _lib.FluteLinear()
     ctypes.memmove(ctypes.byref(c), ctypes.byref(d), ctypes.sizeof(c))
@@ -258,6 +283,7 @@ def _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, down, keep_down,
                                                 H, H, x16)
     del ws
     out["gemv_4096x12288_cache_resident"] = gv.run("cache_resident", gate[:1], keep[:1], I, H, x)
+    out["read_probe_24MiB_cold"] = _read_probe(torch, _lib, dev, keep)
     # (4, 1) two streams: a 1-bit second stream with its own two-entry LUT
     two, keep2 = [], []
     for g_ in gate:

@@ -255,7 +255,8 @@ void flute_release_workspaces(void);
  * The launchers read their tuning and test knobs (FLUTE_GEMV_RW, FLUTE_GEMV_WAVES,
  * FLUTE_GEMV_TABLE_LOG2, FLUTE_GEMV_PREROTATE, FLUTE_GEMV4_PF, FLUTE_GEMV_NO_FAST,
  * FLUTE_GEMV4_WALK, FLUTE_GEMM_ROWS, FLUTE_GEMM_NO_PERM, FLUTE_GEMM_KSPLIT,
- * FLUTE_GEMM_NO_DIRECT, FLUTE_FHT_STEPS) from the environment once per process; this
+ * FLUTE_GEMM_NO_DIRECT, FLUTE_GEMM_NO_LEAN, FLUTE_FHT_STEPS) from the environment once per
+ * process; this
  * re-reads them.
  */
 void flute_reload_tuning(void);
@@ -276,6 +277,17 @@ int flute_workspace_decision(int64_t have_floats, int64_t need_floats, int64_t h
  * returns (uint32)lo | (uint32)hi << 32 for every bit pattern, bit 31 of either half included.
  */
 uint64_t flute_join_address_halves(int32_t lo, int32_t hi);
+
+/*
+ * No upstream counterpart; a measurement aid, not part of the layer.  Reads `bytes` of device
+ * memory once and discards them: `workgroups` workgroups of 256 threads, 16-byte non-temporal
+ * loads, `loads_in_flight` (2, 4 or 8) per thread, the load pattern of the M = 1 kernel without
+ * its table, lookups and sums.  Timed on the bytes of one weight it shows what a single launch of
+ * that size can reach on the device.  sink: 4 bytes of device memory (practically never
+ * written).
+ */
+flute_status flute_read_probe(const void *src, int64_t bytes, int workgroups,
+                              int loads_in_flight, void *sink, void *stream);
 
 /*
  * No upstream counterpart.  Sixteen hex digits of the SHA-256 over the sources the library was

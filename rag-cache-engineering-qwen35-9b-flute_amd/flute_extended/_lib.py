@@ -74,6 +74,7 @@ SYMBOLS = {
     "flute_workspace_decision": (_I, [ctypes.c_int64] * 4 + [_I]),
     "flute_join_address_halves": (ctypes.c_uint64, [ctypes.c_int32, ctypes.c_int32]),
     "flute_build_id": (ctypes.c_char_p, []),
+    "flute_read_probe": (_I, [_P, ctypes.c_int64, _I, _I, _P, _P]),
 }
 
 if not os.path.exists(LIB_PATH):
