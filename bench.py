@@ -195,9 +195,12 @@ class _Gemv:
     def __init__(self, torch, _lib, ctypes, O, dev):
         self.torch, self.lib, self.ct, self.O, self.dev = torch, _lib, ctypes, O, dev
 
-    def run(self, name, descs, keep, N, K, x, xref=None, split=0, launches=None, keep2=None, bits2=0):
+    def run(self, name, descs, keep, N, K, x, xref=None, split=0, launches=None, keep2=None, bits2=0,
+            rows_of=None, wbytes=None):
         """keep[i] = (blob, lut) of descs[i] (keep2: the second stream's); xref: the row the
-        weights see (the rotated x for a fused rotation), default x."""
+        weights see (the rotated x for a fused rotation), default x.  rows_of(tile): the fp64
+        rows of one 128-row tile of weight 0 where they are not the N-grouped dequantisation;
+        wbytes: the bytes of one weight where they are not indices + N-grouped LUT."""
         torch, _lib, ctypes = self.torch, self.lib, self.ct
         act = x.dtype
         code = _lib.BF16 if act == torch.bfloat16 else _lib.F16
@@ -216,6 +219,8 @@ class _Gemv:
         tiles = sorted({0, (N // 128) // 2, N // 128 - 1})
 
         def rows(t):
+            if rows_of is not None:
+                return rows_of(t)
             w = _oracle_rows(self.O, blob, lut, K, t)
             if keep2 is not None:
                 w = w + _oracle_rows(self.O, keep2[0][0], keep2[0][1], K, t, bits2)
@@ -226,8 +231,9 @@ class _Gemv:
         n = launches or max(96, len(descs))
         ms = _time_graph(torch, lambda: [call(i) for i in range(n)])
         us = ms / n * 1e3
-        wbytes = N * K // 2 + (N // GS) * 32
-        if keep2 is not None:
+        given = wbytes is not None
+        wbytes = wbytes if given else N * K // 2 + (N // GS) * 32
+        if keep2 is not None and not given:
             wbytes += N * K * bits2 // 8 + (N // GS) * (2 << bits2)
         res.update({"us_per_call": round(us, 3), "gbs_index_plus_lut": round(wbytes / us / 1e3, 1),
                     "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4),
@@ -296,6 +302,25 @@ def _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, down, keep_down,
         keep2.append((q2, l2))
     out["gemv_4096x12288_two_streams_4_1"] = gv.run("two_streams", two, keep, I, H, x, keep2=keep2, bits2=1)
     del two, keep2
+    # LUT grouped along K: one row of 16 values per (output row, 128-wide K group), [N, K/128, 16]
+    # (a form no upstream artifact has; bytes = indices + that LUT = 37,748,736 at 4096 -> 12288)
+    kluts = [(torch.randn(I, H // 128, 16, device=dev, generator=gen) * 0.02).sort(dim=2).values
+             .to(torch.float16).contiguous() for _ in gate]
+    kds = []
+    for g_, kl in zip(gate, kluts):
+        d = _copy_desc(_lib, ctypes, g_)
+        d.lut1, d.lut_rows, d.k_group, d.lut_dtype = kl.data_ptr(), I * (H // 128), 128, _lib.F16
+        kds.append(d)
+
+    def krows(t):
+        per = (H // 64) * 1024 * 4
+        idx = torch.from_numpy(O.unpack_idxn(keep[0][0][t * per:(t + 1) * per].cpu().numpy(), 128, H, 4)).long()
+        lk = kluts[0][t * 128:(t + 1) * 128].cpu().double()           # [128, K/128, 16]
+        grp = (torch.arange(H) // 128)[None, :].expand(128, H)
+        return lk[torch.arange(128)[:, None].expand(128, H), grp, idx]
+    out["gemv_4096x12288_lut_grouped_along_k"] = gv.run(
+        "k_grouped_lut", kds, keep, I, H, x, rows_of=krows, wbytes=I * H // 2 + I * (H // 128) * 32)
+    del kds, kluts
     # fused rotations
     signs = (torch.randint(0, 2, (H,), device=dev, generator=gen).float() * 2 - 1).contiguous()
     signs_d = (torch.randint(0, 2, (I,), device=dev, generator=gen).float() * 2 - 1).contiguous()

@@ -86,6 +86,17 @@ typedef struct flute_linear {
     int32_t rot_block;     /* 0: rotation over the descending power-of-two segments of K
                               (upstream's transform); > 0: equal blocks of this many
                               columns, each normalised by 1/sqrt(rot_block) */
+    int32_t k_group;       /* 0: the LUT is grouped along N (every upstream artifact).
+                              128: the LUT is grouped along K, one row of 16 values per
+                              (output row, 128-wide K group): lut1 is [N, K/128, 16],
+                              lut_rows = N * K/128, W[n, k] = lut1[n][k / 128][idx[n, k]].
+                              No upstream kernel or artifact has this form; it needs
+                              b1 = 4, b2 = 0, K % 128 == 0 and a 16-byte aligned lut1;
+                              group_size is not read.  Served by flute_gemv,
+                              flute_gemv_noalloc and flute_dequant; every other entry
+                              point refuses it.  (The field takes what were four bytes of
+                              padding at the end of the structure: its size is unchanged,
+                              and a caller that zero-initialises the structure gets 0.) */
 } flute_linear;
 
 /* Library identity and diagnostics. */
@@ -238,7 +249,7 @@ int flute_pick_split(int N, int K);
 int64_t flute_gemv_lds_bytes(const flute_linear *w, int split);
 
 /* Validate a weight descriptor exactly as the launchers do, without touching
- * the device.  mode: 0 = GEMV, 1 = GEMM. */
+ * the device.  mode: 0 = GEMV (accepts k_group = 128), 1 = GEMM (refuses it). */
 flute_status flute_validate(const flute_linear *w, int mode);
 
 /* Release the per-device split-K workspaces (also done at process exit).

@@ -15,12 +15,36 @@ namespace flute {
 
 namespace {
 
+// Residual coefficients: xb[r] = sum_k x[k] * resB[r][k] in fp32, one workgroup
+// per residual row, x taken as given (already rotated).  A thread-strided sum
+// followed by a fixed-order tree: deterministic.
+__global__ void __launch_bounds__(256) residual_coeff_kernel(const uint16_t *x,
+                                                             const uint16_t *resB, float *xb,
+                                                             int K, int act_bf16) {
+    __shared__ float part[256];
+    const uint16_t *row = resB + (size_t)blockIdx.x * K;
+    float s = 0.0f;
+    for (int k = threadIdx.x; k < K; k += 256) {
+        const float a = act_bf16 ? bf2f(x[k]) : h2f(x[k]);
+        const float b = act_bf16 ? bf2f(row[k]) : h2f(row[k]);
+        s = fmaf(a, b, s);
+    }
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int step = 128; step > 0; step >>= 1) {
+        if ((int)threadIdx.x < step) part[threadIdx.x] += part[threadIdx.x + step];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) xb[blockIdx.x] = part[0];
+}
+
 int entries_log2(int bits) { return bits == 3 ? 6 : 8; }
 int entry_bytes_log2(int bits) { return bits >= 3 ? 2 : (bits == 2 ? 3 : 4); }
 
 struct Plan {
     GemvParams p;
     int pair;               // 10 * b1 + b2 when the widths are a pair the lean kernel serves with two tables, else 0
+    bool k_group;           // the LUT is grouped along K (single weight, lean kernel only)
     size_t lds_bytes;
     int grid_x;
     int threads;
@@ -113,7 +137,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     FLUTE_REQUIRE(act_dtype == FLUTE_F16 || act_dtype == FLUTE_BF16, FLUTE_ERR_INVALID,
                   "%s: activations must be float16 or bfloat16", who);
     for (int i = 0; i < count; ++i) {
-        flute_status st = validate_linear(&segs[i], 0, who);
+        flute_status st = validate_linear(&segs[i], count == 1 && !silu_mul ? kModeKGroupOk : 0, who);
         if (st != FLUTE_OK) return st;
         FLUTE_REQUIRE(outs[i] != nullptr, FLUTE_ERR_INVALID, "%s: output %d is NULL", who, i);
         FLUTE_REQUIRE(((uintptr_t)outs[i] & 1) == 0, FLUTE_ERR_INVALID,
@@ -141,6 +165,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     FLUTE_REQUIRE(split <= 0 || G % split == 0, FLUTE_ERR_INVALID,
                   "%s: split %d must divide K/64 = %d", who, split, G);
 
+    const int split_in = split;
     GemvParams &p = plan->p;
     std::memset(&p, 0, sizeof(p));
     int rows = 0;
@@ -151,6 +176,42 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     // (the library's own K split was measured on single weights only: merged gate/up launches
     // split when the caller asks for it)
     choose_shape(rows, G, split, &rw, &split, &waves, !rotated && !silu_mul);
+    const bool k_group = segs[0].k_group != 0;
+    if (k_group) {
+        // Only the lean kernel serves this form: four or eight wavefronts, each with an even
+        // number (two at least) of loads of 32 / rw tiles.  The workgroup stages its LUT rows in
+        // LDS, 32 bytes per (row, K group), at most kKGroupPieces 16-byte pieces per thread, whole
+        // K groups per split.  The shape chosen above is kept where it fits; else wider slices or
+        // another wavefront count; else, where the library chooses the split, a larger one.
+        auto ok = [&](int sp, int rw_, int wv) {
+            if (G % sp || (G / sp) % 2 || (G / sp) % (32 / rw_)) return false;
+            const int units = (G / sp) / (32 / rw_);
+            if (!(wv == 4 || (wv == 8 && rw_ <= 16)) || units % wv) return false;
+            const int u = units / wv;
+            return u >= 2 && u % 2 == 0 &&
+                   (long)rw_ * (G / sp / 2) * 2 <= (long)kKGroupPieces * wv * 64;
+        };
+        auto settle = [&](int sp) {
+            if (ok(sp, rw, waves)) return true;
+            for (int r = rw; r <= 32; r *= 2)
+                for (int wv : {4, 8})
+                    if (ok(sp, r, wv)) {
+                        rw = r;
+                        waves = wv;
+                        return true;
+                    }
+            return false;
+        };
+        bool done = settle(split);
+        for (int sp = split * 2; !done && split_in <= 0 && sp <= G / 2 && G % sp == 0; sp *= 2) {
+            choose_shape(rows, G, sp, &rw, &split, &waves, false);
+            done = settle(split);
+        }
+        FLUTE_REQUIRE(done, FLUTE_ERR_UNSUPPORTED,
+                      "%s: K=%d at split %d does not divide into the loads of the kernel that serves "
+                      "a LUT grouped along K (K/split must be a multiple of 512 whose LUT rows fit a "
+                      "workgroup's staging); try another split", who, K, split);
+    }
     FLUTE_REQUIRE((G / split) % (32 / rw) == 0, FLUTE_ERR_UNSUPPORTED,
                   "%s: K/64/split = %d is not a whole number of wavefront loads", who, G / split);
     const int gs_tiles = G / split;
@@ -194,7 +255,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
         sg.out = (uint16_t *)outs[i];
         sg.N = w.N;
         sg.R = w.R;
-        sg.gs = w.group_size;
+        sg.gs = k_group ? 128 : w.group_size;       // (a LUT grouped along K: group_size is not read)
         sg.lut_rows = w.lut_rows;
         sg.nstreams = w.b2 > 0 ? 2 : 1;
         sg.n0 = n0;
@@ -234,7 +295,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
             sg.awq = w.awq;
             any_fused_rot |= w.signs != nullptr;
         }
-        const int ngrp_log2 = w.group_size >= 128 ? 0 : ilog2(128 / w.group_size);
+        const int ngrp_log2 = k_group || w.group_size >= 128 ? 0 : ilog2(128 / w.group_size);
         for (int st = 0; st < sg.nstreams; ++st) {
             GemvStream &gs = sg.st[st];
             gs.q = (const uint8_t *)(st ? w.q2 : w.q1);
@@ -243,8 +304,10 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
             int es = budget - entries_log2(gs.bits) - ngrp_log2;
             if (es > 7) es = 7;             // 32 replicas cover the 32 LDS banks
             if (es < entry_bytes_log2(gs.bits)) es = entry_bytes_log2(gs.bits);
+            if (k_group) es = 7;            // (no table: the lean kernel's LUT rows, sized below)
             gs.es = es;
-            const size_t tb = ((size_t)1 << (entries_log2(gs.bits) + es)) << ngrp_log2;
+            const size_t tb = k_group ? (size_t)(kc / 128) * (rw * 32 + (rw / 8) * 32)
+                                      : ((size_t)1 << (entries_log2(gs.bits) + es)) << ngrp_log2;
             if (tb > tab_bytes) tab_bytes = tb;
         }
     }
@@ -280,7 +343,8 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     // side (4^b entries of 128 bytes each).  Decided here because it sets the table region;
     // the launcher may still send the launch to the general kernel, which needs less.
     plan->pair = 0;
-    {
+    plan->k_group = k_group;
+    if (!k_group) {
         int b1 = segs[0].b1, b2 = 0;
         bool ok = true;
         for (int i = 0; i < count; ++i) {
@@ -458,6 +522,16 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
     for (int i = 0; i < plan.p.nsegs; ++i)
         for (int st = 0; st < plan.p.seg[i].nstreams; ++st)
             luts_aligned &= ((uintptr_t)plan.p.seg[i].st[st].lut & 3) == 0;
+    if (plan.k_group) {
+        // only the lean kernel knows this form: no general-kernel route
+        const int pf = pick_prefetch(plan, nw);
+        FLUTE_REQUIRE(pf != 0 && (nw == 4 || (nw == 8 && plan.p.lpg_log2 <= 5)), FLUTE_ERR_UNSUPPORTED,
+                      "flute_gemv: K=%d at split %d with %d-row workgroups of %d wavefronts does not "
+                      "divide into the loads of the kernel that serves a LUT grouped along K; try "
+                      "another split", plan.p.K, plan.p.split, 1 << (plan.p.lpg_log2 - 1), nw);
+        plan.p.slices = 0;
+        return launch_gemv_kgroup(plan.p, plan.grid_x, nw, pf, plan.lds_bytes, BF16, stream);
+    }
     if (bits == 4 && one_group && one_input && es == 7 && (nw == 4 || nw == 8) && luts_aligned &&
         pick_prefetch(plan, nw) != 0 && tuning().gemv_no_fast == 0) {
         switch (plan.p.lpg_log2) {

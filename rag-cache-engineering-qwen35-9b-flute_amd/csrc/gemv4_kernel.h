@@ -187,6 +187,9 @@ __device__ __forceinline__ void rotate_piece(uint4 &v, const float (&sg)[8], con
     v = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// A LUT grouped along K: 16-byte pieces of LUT rows a thread stages at most.
+constexpr int kKGroupPieces = 8;
+
 // LPGL = log2(lanes per 64-k tile) = log2(2 * rows per workgroup): 4, 5, 6.
 // NW   = wavefronts per workgroup (4 or 8).
 // PF   = index loads a lane keeps in flight (2 or 4).  The host picks a PF that
@@ -201,7 +204,14 @@ __device__ __forceinline__ void rotate_piece(uint4 &v, const float (&sg)[8], con
 // pairs of deployed artifacts, (3, 3)) has small tables: both are built before an output's first
 // loop (the first at offset 0, the second behind it) and the two K loops run back to back, with
 // no barrier and no table build between them.
-template <int LPGL, int NW, int PF, bool BF16, bool WALK = false, int BA = 4, int BB = 4>
+// KG: the LUT is grouped along K instead of along N: one row of sixteen values per (output row,
+// 128-wide K group), W[n, k] = LUT[n][k / 128][idx[n, k]] (a variant no upstream artifact has;
+// single weight, one 4-bit stream).  No pair table then (it would be 1 KB per 128 weights): the
+// workgroup stages the LUT rows of its row slice and K range in LDS, group-major with the rows
+// of a group 32 bytes apart, and a weight is one 16-bit read at (code * 2) in its row.  A row is
+// eight dwords on eight different banks and equal dwords are broadcast, so the lanes of a lookup
+// (two rows per wavefront instruction, padded onto different banks) never conflict.
+template <int LPGL, int NW, int PF, bool BF16, bool WALK = false, int BA = 4, int BB = 4, bool KG = false>
 __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int ES = 7;
@@ -222,6 +232,8 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     static_assert(!WALK || NW == 4, "the alternating sum areas of a walking grid are sized for four wavefronts");
     constexpr bool TWO = !(BA == 4 && BB == 4);     // two resident tables
     static_assert(!TWO || !WALK, "walking grids: the (4, 4) kernel");
+    static_assert(!KG || (!TWO && !WALK), "K-grouped LUTs: one 4-bit stream, one slice per workgroup");
+    constexpr int KG_GROUP = RW * 32 + (RW / 8) * 32;   // LDS bytes of one K group's rows
     constexpr int TAB_A = (1 << (2 * BA)) * STRIDE; // bytes of the first table
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
@@ -341,8 +353,45 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             for (int k = 0; k < CHUNKS; ++k) *(uint4 *)(ent + (((k + tid) & (CHUNKS - 1)) << 4)) = v4;
         }
     };
+    // K-grouped LUT: the rows of this slice for the K groups of this launch's K range, 16 bytes
+    // per piece, consecutive threads on consecutive pieces of a row in memory.  At most eight
+    // pieces per thread (the host checks); a thread beyond the end re-reads piece 0.
+    constexpr int KG_MAX = kKGroupPieces;
+    uint4 slab_v[KG ? KG_MAX : 1];
+    const int kg_groups = kc >> 7;                  // K groups of the range
+    const int kg_pieces = RW * kg_groups * 2;
+    auto slab_issue = [&]() {
+        if constexpr (KG) {
+            const int t0 = sl / SPT, cg0 = (sl % SPT) * (RW >> 3);
+            const uint16_t *lutk = kp->seg[si0].st[0].lut;
+#pragma unroll
+            for (int i = 0; i < KG_MAX; ++i) {
+                int idx = tid + i * NT;
+                if (idx >= kg_pieces) idx = 0;
+                const int r = idx / (kg_groups * 2), pc = idx % (kg_groups * 2);
+                const int n = t0 * 128 + row_of(cg0 + (r >> 3), r & 7);
+                slab_v[i] = *(const uint4 *)(lutk + (((size_t)n * (p.K >> 7) + (k0 >> 7)) << 4) + pc * 8);
+            }
+        }
+    };
+    auto slab_write = [&]() {
+        if constexpr (KG) {
+#pragma unroll
+            for (int i = 0; i < KG_MAX; ++i) {
+                const int idx = tid + i * NT;
+                if (idx < kg_pieces) {
+                    const int r = idx / (kg_groups * 2), pc = idx % (kg_groups * 2);
+                    *(uint4 *)(lds + (pc >> 1) * KG_GROUP + r * 32 + (r >> 3) * 32 + (pc & 1) * 16) = slab_v[i];
+                }
+            }
+        }
+    };
     // the tables of one output: the first stream's, and (two resident tables) the second's
     auto write_tables = [&](const uint32_t (&rowA)[8], const uint32_t (&rowB)[8], bool second) {
+        if constexpr (KG) {
+            slab_write();
+            return;
+        }
         if constexpr (BA == 4) write_table(rowA);
         else write_small_table(rowA, std::integral_constant<int, BA>(), 0u);
         if constexpr (TWO) {
@@ -386,7 +435,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const uint16_t *lut;
     pass_ptrs(sl, 0, 0, qrow, lut);
     uint32_t lrow[8], lrowB[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
-    load_lut_row<BA>(lut, lrow);
+    if constexpr (!KG) load_lut_row<BA>(lut, lrow);
     bool second0 = false;                           // two tables: this output has a second stream
     if constexpr (TWO) {
         second0 = kp->seg[si0].nstreams == 2;
@@ -446,6 +495,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 if (staged_awq) load_f8(staged_awq, k0 + (j >= 0 ? j : 0), scv[i]);
             }
         }
+        slab_issue();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int n = 0; n < PF0; ++n) {
@@ -510,6 +560,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 stage8(j, !convert ? v : finite ? bf16_to_f16_top8(v, adj) : bf16_to_f16_scaled8(v, 0));
             }
         }
+        slab_issue();
         write_tables(lrow, lrowB, second0);
         __builtin_amdgcn_sched_barrier(0);
         first_units(qrow, q, 0);
@@ -522,6 +573,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             __builtin_amdgcn_sched_barrier(0);
         }
         xshift = stage_x<BF16>(p, staged_x, staged_signs, staged_awq, lds, k0, kc, tid, NT);
+        slab_issue();
         write_tables(lrow, lrowB, second0);
         __builtin_amdgcn_sched_barrier(0);
         first_units(qrow, q, PF0);
@@ -589,12 +641,23 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     };
     // per row group v, eight lookups feed two matrix products; pair pp = v * 4 + d * 2 + s2 of a
     // quarter, an operand is (s2 = 0, 1) of both units
-    auto unit_pair = [&](const auto &qa, const auto &qb, gv_u4_t Bop, uint32_t tslot, auto width) {
+    // (K-grouped LUT: ga, gb = LDS byte offsets of the two units' K groups plus this lane's rows)
+    typedef const __attribute__((address_space(3))) uint16_t *LdsHalf;
+    auto unit_pair = [&](const auto &qa, const auto &qb, gv_u4_t Bop, uint32_t tslot, auto width,
+                         uint32_t ga = 0, uint32_t gb = 0) {
         constexpr int B = decltype(width)::value;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            auto look = [&](const IdxQuarter<B> &qq, int j) -> uint32_t {
-                if constexpr (B == 4 && !TWO) {
+            auto look = [&](const IdxQuarter<B> &qq, int j, uint32_t goff = 0) -> uint32_t {
+                if constexpr (KG) {
+                    // byte j of dword v: rows a = 2 v + (j >> 1); the two codes of the pair are
+                    // two 16-bit reads in that row of the unit's K group
+                    const uint32_t base = goff + (uint32_t)((2 * v + (j >> 1)) * 32);
+                    const uint32_t c0 = __builtin_amdgcn_ubfe(qq.d[v], 8 * j, 4);
+                    const uint32_t c1 = __builtin_amdgcn_ubfe(qq.d[v], 8 * j + 4, 4);
+                    const uint32_t lo = *(LdsHalf)((c0 << 1) + base), hi = *(LdsHalf)((c1 << 1) + base);
+                    return lo | (hi << 16);
+                } else if constexpr (B == 4 && !TWO) {
                     // a whole byte of dword v; byte 0: shift, then one and-or (the slot lies
                     // below the stride, the table at offset 0)
                     const uint32_t wq = qq.d[v];
@@ -604,11 +667,17 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                     return *(LdsWord)((quarter_code<B>(qq, v * 4 + j) << ES) + tslot);
                 }
             };
-            const gv_u4_t A0 = {look(qa, 0), look(qa, 1), look(qb, 0), look(qb, 1)};
-            const gv_u4_t A1 = {look(qa, 2), look(qa, 3), look(qb, 2), look(qb, 3)};
+            const gv_u4_t A0 = {look(qa, 0, ga), look(qa, 1, ga), look(qb, 0, gb), look(qb, 1, gb)};
+            const gv_u4_t A1 = {look(qa, 2, ga), look(qa, 3, ga), look(qb, 2, gb), look(qb, 3, gb)};
             acc[v * 2] = gv_mfma<BF16>(A0, Bop, acc[v * 2]);
             acc[v * 2 + 1] = gv_mfma<BF16>(A1, Bop, acc[v * 2 + 1]);
         }
+    };
+    // K-grouped LUT: LDS offset of unit m's K group (tile (w + m NW) GPI + gsub of the range, two
+    // tiles per group) plus this lane's first row (chunk group cgl: eight rows and one pad).
+    auto kg_off = [&](int m) -> uint32_t {
+        if constexpr (!KG) return 0u;
+        return (uint32_t)((((w + m * NW) * GPI + gsub) >> 1) * KG_GROUP + cgl * (8 * 32 + 32));
     };
     // The K range of one stream of width B held in qc, refilled from qcur; the last group's
     // registers are refilled with the first loads of what follows: a stream of width BN from
@@ -623,7 +692,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 #pragma unroll
             for (int n = 0; n < PF; n += 2) {
                 const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
-                unit_pair(qc[n], qc[n + 1], Bop, tslot, width);
+                unit_pair(qc[n], qc[n + 1], Bop, tslot, width, kg_off(nb + n), kg_off(nb + n + 1));
                 __builtin_amdgcn_sched_barrier(0);
                 qc[n] = load_idx<B>(qcur + (size_t)(nb + n + PF) * step_c + lane_c);
                 qc[n + 1] = load_idx<B>(qcur + (size_t)(nb + n + 1 + PF) * step_c + lane_c);
@@ -635,7 +704,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 #pragma unroll
             for (int n = 0; n < PF; n += 2) {
                 const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
-                unit_pair(qc[n], qc[n + 1], Bop, tslot, width);
+                unit_pair(qc[n], qc[n + 1], Bop, tslot, width, kg_off(nb + n), kg_off(nb + n + 1));
                 __builtin_amdgcn_sched_barrier(0);
                 qn[n] = load_idx<BN>(qnext + (size_t)n * step_n + lane_n);
                 qn[n + 1] = load_idx<BN>(qnext + (size_t)(n + 1) * step_n + lane_n);
@@ -645,7 +714,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 #pragma unroll
             for (int n = 0; n < PF; n += 2) {
                 const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
-                unit_pair(qc[n], qc[n + 1], Bop, tslot, width);
+                unit_pair(qc[n], qc[n + 1], Bop, tslot, width, kg_off(nb + n), kg_off(nb + n + 1));
             }
         }
         if (!has_next) __builtin_amdgcn_s_setprio(0);
@@ -817,5 +886,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 
     if (owner) finish_rows(sl, yv);
 }
+
+// The launch of the K-grouped instantiations (its own translation unit).  nw: wavefronts per
+// workgroup, pf: loads in flight (pick as for the lean kernel), p.lpg_log2 in 4..6.
+flute_status launch_gemv_kgroup(const GemvParams &p, int grid_x, int nw, int pf, size_t lds_bytes,
+                                bool lut_bf16, hipStream_t stream);
 
 }  // namespace flute

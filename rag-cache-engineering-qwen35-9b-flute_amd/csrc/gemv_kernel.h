@@ -1098,27 +1098,4 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     }
 }
 
-// Residual coefficients: xb[r] = sum_k x[k] * resB[r][k] in fp32, one workgroup
-// per residual row, x taken as given (already rotated).  A thread-strided sum
-// followed by a fixed-order tree: deterministic.
-__global__ void __launch_bounds__(256) residual_coeff_kernel(const uint16_t *x,
-                                                             const uint16_t *resB, float *xb,
-                                                             int K, int act_bf16) {
-    __shared__ float part[256];
-    const uint16_t *row = resB + (size_t)blockIdx.x * K;
-    float s = 0.0f;
-    for (int k = threadIdx.x; k < K; k += 256) {
-        const float a = act_bf16 ? bf2f(x[k]) : h2f(x[k]);
-        const float b = act_bf16 ? bf2f(row[k]) : h2f(row[k]);
-        s = fmaf(a, b, s);
-    }
-    part[threadIdx.x] = s;
-    __syncthreads();
-    for (int step = 128; step > 0; step >>= 1) {
-        if ((int)threadIdx.x < step) part[threadIdx.x] += part[threadIdx.x + step];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) xb[blockIdx.x] = part[0];
-}
-
 }  // namespace flute

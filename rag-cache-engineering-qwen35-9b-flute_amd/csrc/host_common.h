@@ -7,7 +7,9 @@
 namespace flute {
 
 // Shape/size/alignment contract of one weight (no device access).
-// mode: 0 = GEMV, 1 = GEMM / dequant.
+// mode: 0 = GEMV, 1 = GEMM / dequant; | kModeKGroupOk where the entry point serves a LUT
+// grouped along K (flute_linear.k_group).
+constexpr int kModeKGroupOk = 0x100;
 flute_status validate_linear(const flute_linear *w, int mode, const char *who);
 
 // Split-K workspace of the current device: `floats` fp32 partial sums and

@@ -47,10 +47,30 @@ flute_status validate_linear(const flute_linear *w, int mode, const char *who) {
     FLUTE_REQUIRE(aligned(w->q1, 16), FLUTE_ERR_INVALID,
                   "%s: stream-1 indices must be 16-byte aligned", who);
     FLUTE_REQUIRE(aligned(w->lut1, 2), FLUTE_ERR_INVALID, "%s: lut misaligned", who);
-    const int rows = (w->N + gs - 1) / gs;
-    FLUTE_REQUIRE(w->lut_rows == rows, FLUTE_ERR_INVALID,
-                  "%s: lut must be [ceil(N/group_size), 2^bitwidth] = [%d, %d] (got %d rows)", who,
-                  rows, 1 << w->b1, w->lut_rows);
+    if (w->k_group != 0) {
+        // the LUT grouped along K: [N, K/128, 16]
+        FLUTE_REQUIRE((mode & kModeKGroupOk) != 0, FLUTE_ERR_UNSUPPORTED,
+                      "%s: a LUT grouped along K (k_group = %d) is served by flute_gemv, "
+                      "flute_gemv_noalloc and flute_dequant only", who, w->k_group);
+        FLUTE_REQUIRE(w->k_group == 128, FLUTE_ERR_INVALID,
+                      "%s: k_group must be 0 (LUT grouped along N) or 128 (got %d)", who, w->k_group);
+        FLUTE_REQUIRE(w->b1 == 4 && w->b2 == 0, FLUTE_ERR_UNSUPPORTED,
+                      "%s: a LUT grouped along K has one 4-bit stream (got b1=%d, b2=%d)", who, w->b1,
+                      w->b2);
+        FLUTE_REQUIRE(w->K % 128 == 0, FLUTE_ERR_INVALID,
+                      "%s: a LUT grouped along K needs K %% 128 == 0 (got K=%d)", who, w->K);
+        const int64_t krows = (int64_t)w->N * (w->K / 128);
+        FLUTE_REQUIRE(krows <= INT32_MAX && w->lut_rows == (int32_t)krows, FLUTE_ERR_INVALID,
+                      "%s: a LUT grouped along K must be [N, K/128, 16] = %lld rows (got %d)", who,
+                      (long long)krows, w->lut_rows);
+        FLUTE_REQUIRE(aligned(w->lut1, 16), FLUTE_ERR_INVALID,
+                      "%s: a LUT grouped along K must be 16-byte aligned (read 16 bytes at a time)", who);
+    } else {
+        const int rows = (w->N + gs - 1) / gs;
+        FLUTE_REQUIRE(w->lut_rows == rows, FLUTE_ERR_INVALID,
+                      "%s: lut must be [ceil(N/group_size), 2^bitwidth] = [%d, %d] (got %d rows)", who,
+                      rows, 1 << w->b1, w->lut_rows);
+    }
     if (w->b2 > 0) {
         FLUTE_REQUIRE(w->q2 != nullptr && w->lut2 != nullptr, FLUTE_ERR_INVALID,
                       "%s: a second stream needs both indices2 and lut2", who);
@@ -245,14 +265,15 @@ const Tuning &tuning() {
 
 extern "C" {
 
-int flute_abi_version(void) { return 1; }
+int flute_abi_version(void) { return 2; }
 
 const char *flute_last_error(void) { return flute::g_error; }
 
 const char *flute_target_arch(void) { return "gfx950"; }
 
 flute_status flute_validate(const flute_linear *w, int mode) {
-    return flute::validate_linear(w, mode, "flute_validate");
+    // (mode 0, the GEMV, serves a LUT grouped along K; the GEMM does not)
+    return flute::validate_linear(w, mode == 0 ? flute::kModeKGroupOk : (mode & 0xff), "flute_validate");
 }
 
 void flute_reload_tuning(void) {

@@ -489,6 +489,75 @@ def dequant_idxn(indices, lut, N: int, K: int, bitwidth: int, group_size: int):
 
 
 # ---------------------------------------------------------------------------
+# LUT grouped along K (no upstream counterpart: no upstream kernel or artifact has this
+# form; one 16-entry row per (output row, 128-wide K group))
+# ---------------------------------------------------------------------------
+
+K_GROUP = 128
+
+
+def _describe_kgroup(who: str, A: torch.Tensor, K: int, indices, lut, bias=None, signs=None,
+                     awq=None, rot_block: int = 0):
+    """Descriptor of a weight whose LUT is [N, K/128, 16]: W[n, k] = lut[n, k // 128, idx[n, k]],
+    indices the 4-bit idxN blob.  The checks of _describe where they apply, then the form's own."""
+    if lut.dim() != 3 or lut.shape[2] != 16:
+        _fail(f"{who}: a LUT grouped along K must be [N, K/{K_GROUP}, 16] (got {tuple(lut.shape)})")
+    if K % K_GROUP != 0:
+        _fail(f"{who}: a LUT grouped along K needs K % {K_GROUP} == 0 (got K={K})")
+    N = int(lut.shape[0])
+    if lut.shape[1] != K // K_GROUP:
+        _fail(f"{who}: a LUT grouped along K must be [N, K/{K_GROUP}, 16] = "
+              f"[{N}, {K // K_GROUP}, 16] (got {tuple(lut.shape)})")
+    e8 = torch.empty(0, dtype=torch.uint8, device=A.device)
+    e16 = torch.empty(0, dtype=A.dtype, device=A.device)
+    # the shared checks see a stand-in LUT of the N-grouped shape for the same N
+    n_blob = indices.numel() // max(K // 2, 1)
+    if n_blob != N:
+        _fail(f"{who}: the blob holds N={n_blob} rows, the LUT {N}")
+    stand_in = lut.reshape(-1, 16)[: (N + 127) // 128]
+    w, N2, keep = _describe(who, A, K, indices, stand_in, 4, e8, e16, 0, e16, e16,
+                            bias if bias is not None else e16, 128, signs, awq, rot_block)
+    if N2 != N:
+        _fail(f"{who}: the blob holds N={N2} rows, the LUT {N}")
+    if not lut.is_contiguous():
+        _fail(f"{who}: the LUT must be contiguous")
+    lut = _aligned16(lut)
+    w.lut1 = lut.data_ptr()
+    w.lut_rows = N * (K // K_GROUP)
+    w.k_group = K_GROUP
+    return w, N, (keep, lut)
+
+
+def qgemm_gemv_kgroup(A, indices, lut, bias=None, signs=None, s=None, split: int = 0,
+                      rot_block: int = 0):
+    """Decode GEMV over a weight whose LUT is grouped along K: y[1, N] = A[1, K] . W^T with
+    W[n, k] = lut[n, k // 128, idx[n, k]] (lut [N, K/128, 16], indices the 4-bit idxN blob).
+    signs (and s) select the fused rotation of A as in qgemm_gemv_fht_stream."""
+    who = "qgemm_gemv_kgroup"
+    M, K = _check_2d_input(who, A, need_m1=True)
+    w, N, keep = _describe_kgroup(who, A, K, indices, lut, bias, signs, s, rot_block)
+    A = _aligned16(A)
+    with _on_device_of(A):
+        C = torch.empty((1, N), dtype=A.dtype, device=A.device)
+        check(lib.flute_gemv(ctypes.byref(w), A.data_ptr(), C.data_ptr(), _ACT[A.dtype],
+                             int(split), _stream_of(A)))
+    del keep
+    return C
+
+
+def dequant_kgroup(indices, lut, K: int):
+    """Dense [N, K] dump of a weight whose LUT is grouped along K, in the LUT's dtype (bit exact)."""
+    who = "dequant_kgroup"
+    A = torch.empty((1, int(K)), dtype=lut.dtype, device=lut.device)
+    w, N, keep = _describe_kgroup(who, A, int(K), indices, lut)
+    with _on_device_of(A):
+        W = torch.empty((N, int(K)), dtype=lut.dtype, device=lut.device)
+        check(lib.flute_dequant(ctypes.byref(w), 1, W.data_ptr(), _stream_of(A)))
+    del keep
+    return W
+
+
+# ---------------------------------------------------------------------------
 # rotation                                  (src/bindings.cpp:386-399 upstream)
 # ---------------------------------------------------------------------------
 

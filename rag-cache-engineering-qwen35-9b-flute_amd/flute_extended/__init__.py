@@ -47,6 +47,7 @@ from ._C import qgemm_gemv_multi as _qgemm_gemv_multi
 from ._C import qgemm_gemv_mlp as _qgemm_gemv_mlp
 from ._C import dequant_idxn
 from ._C import embedding_gather
+from ._C import qgemm_gemv_kgroup, dequant_kgroup
 
 Backend = Literal["debug_simple", "cutlass_dense", "cutlass_streaming", "auto"]
 IndicesLayout = Literal["idx1", "idx2", "idx3", "idx4"]
@@ -401,4 +402,5 @@ __all__ = [
     "gemv_multi_supported", "qgemm_gemv_mlp", "gemv_mlp_available", "gemv_mlp_supported",
     "gemv_split_hint", "GEMV_SPLITK_PAIRS", "GEMV_SPLITK_GROUP_SIZES",
     "GEMV_SPLITK_MAX_RESIDUAL_RANK", "dequant_idxn", "embedding_gather",
+    "qgemm_gemv_kgroup", "dequant_kgroup",
 ]

@@ -44,6 +44,7 @@ class FluteLinear(ctypes.Structure):
         ("group_size", ctypes.c_int32),
         ("lut_dtype", ctypes.c_int32),
         ("rot_block", ctypes.c_int32),
+        ("k_group", ctypes.c_int32),
     ]
 
 

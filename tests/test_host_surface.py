@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.flute_abi_version() == 1
+    assert lib.flute_abi_version() == 2
     assert _lib.lib.flute_target_arch() == b"gfx950"
 
 
@@ -58,9 +58,10 @@ def test_loaded_library_is_the_tree_s_build():
 
 
 def test_struct_layout_matches_header():
-    # 9 pointers, 2 int64, 9 int32 -> 8*9 + 16 + 36 = 124, padded to 128
+    # 9 pointers, 2 int64, 10 int32 -> 8*9 + 16 + 40 = 128 (k_group took the tail padding)
     assert ctypes.sizeof(_lib.FluteLinear) == 128
     assert _lib.FluteLinear.q1_bytes.offset == 72 and _lib.FluteLinear.lut_rows.offset == 88
+    assert _lib.FluteLinear.rot_block.offset == 120 and _lib.FluteLinear.k_group.offset == 124
 
 
 def _desc(N=256, K=128, b1=4, b2=0, gs=128, R=0, **over):
@@ -111,6 +112,45 @@ def test_c_validation(over, code):
     assert _lib.lib.flute_validate(ctypes.byref(w), 0) == code
     if code != _lib.FLUTE_OK:
         assert _lib.last_error()
+
+
+def _kdesc(N=256, K=512, **over):
+    """A weight whose LUT is grouped along K: [N, K/128, 16]."""
+    over = dict({"k_group": 128, "lut_rows": N * (K // 128)}, **over)
+    return _desc(N=N, K=K, **over)
+
+
+@pytest.mark.parametrize("over,mode,code", [
+    ({}, 0, _lib.FLUTE_OK),
+    ({}, 1, _lib.FLUTE_ERR_UNSUPPORTED),                  # the GEMM does not serve the form
+    ({"k_group": 64}, 0, _lib.FLUTE_ERR_INVALID),
+    ({"k_group": 256}, 0, _lib.FLUTE_ERR_INVALID),
+    ({"lut_rows": 2}, 0, _lib.FLUTE_ERR_INVALID),         # the N-grouped row count
+    ({"b1": 3}, 0, _lib.FLUTE_ERR_UNSUPPORTED),
+    ({"b2": 1, "q2": 4096, "lut2": 4096}, 0, _lib.FLUTE_ERR_UNSUPPORTED),
+    ({"K": 192, "lut_rows": 256}, 0, _lib.FLUTE_ERR_INVALID),      # K not whole groups
+    ({"lut1": 4096 + 8}, 0, _lib.FLUTE_ERR_INVALID),      # read 16 bytes at a time
+    ({"group_size": 64}, 0, _lib.FLUTE_OK),               # not read
+])
+def test_c_validation_of_a_lut_grouped_along_k(over, mode, code):
+    w = _kdesc(**over)
+    assert _lib.lib.flute_validate(ctypes.byref(w), mode) == code
+    if code != _lib.FLUTE_OK:
+        assert _lib.last_error()
+
+
+def test_lut_grouped_along_k_is_refused_outside_the_single_gemv():
+    w = _kdesc()
+    assert _lib.lib.flute_gemm(ctypes.byref(w), 4096, 4096, 4, 512, 256, 0, None) == _lib.FLUTE_ERR_UNSUPPORTED
+    assert "grouped along K" in _lib.last_error()
+    assert _lib.lib.flute_embedding(ctypes.byref(w), 4096, 1, 4096, None) == _lib.FLUTE_ERR_UNSUPPORTED
+    g, u = _kdesc(), _kdesc()
+    assert _lib.lib.flute_gemv_mlp(ctypes.byref(g), ctypes.byref(u), 4096, 4096, 0, 0, None) \
+        == _lib.FLUTE_ERR_UNSUPPORTED
+    # the single GEMV plans it: LDS = LUT rows of a workgroup + activations + sums
+    assert _lib.lib.flute_gemv_lds_bytes(ctypes.byref(w), 0) > 0
+    # a split that cuts a K group in two is refused (K = 512: split 8 leaves 64 columns)
+    assert _lib.lib.flute_gemv_lds_bytes(ctypes.byref(w), 8) == 0
 
 
 def test_c_entry_points_refuse_before_touching_the_device():
