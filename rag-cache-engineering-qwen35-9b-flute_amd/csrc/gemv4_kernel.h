@@ -358,30 +358,52 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // pieces per thread (the host checks); a thread beyond the end re-reads piece 0.
     constexpr int KG_MAX = kKGroupPieces;
     uint4 slab_v[KG ? KG_MAX : 1];
-    const int kg_groups = kc >> 7;                  // K groups of the range
-    const int kg_pieces = RW * kg_groups * 2;
+    const int kg_row_pieces = (kc >> 7) * 2;        // 16-byte pieces of one row's K groups of the range
+    const int kg_pieces = RW * kg_row_pieces;
+    // piece tid + i NT = (row kg_r, piece kg_pc of the row), stepped without a division per piece:
+    // one division for the thread's first piece, the step NT = (kg_dr rows, kg_dp pieces) is uniform
+    int kg_r = 0, kg_pc = 0;
+    const int kg_dr = __builtin_amdgcn_readfirstlane(NT / max(kg_row_pieces, 1));
+    const int kg_dp = NT - kg_dr * kg_row_pieces;
     auto slab_issue = [&]() {
         if constexpr (KG) {
             const int t0 = sl / SPT, cg0 = (sl % SPT) * (RW >> 3);
-            const uint16_t *lutk = kp->seg[si0].st[0].lut;
+            const uint16_t *lutk = kp->seg[si0].st[0].lut + ((size_t)(k0 >> 7) << 4);
+            const int row_stride = (p.K >> 7) << 4;             // 16-bit values per output row
+            int r = tid / kg_row_pieces, pc = tid - r * kg_row_pieces;
+            kg_r = r;
+            kg_pc = pc;
 #pragma unroll
             for (int i = 0; i < KG_MAX; ++i) {
-                int idx = tid + i * NT;
-                if (idx >= kg_pieces) idx = 0;
-                const int r = idx / (kg_groups * 2), pc = idx % (kg_groups * 2);
-                const int n = t0 * 128 + row_of(cg0 + (r >> 3), r & 7);
-                slab_v[i] = *(const uint4 *)(lutk + (((size_t)n * (p.K >> 7) + (k0 >> 7)) << 4) + pc * 8);
+                if (i * NT < kg_pieces) {                       // (uniform: whole rounds beyond the end are skipped)
+                    const bool in = r < RW;                     // (the last round: threads beyond the end re-read piece 0)
+                    const int rr = in ? r : 0, pp = in ? pc : 0;
+                    const int n = t0 * 128 + row_of(cg0 + (rr >> 3), rr & 7);
+                    slab_v[i] = *(const uint4 *)(lutk + (size_t)n * row_stride + pp * 8);
+                    r += kg_dr;
+                    pc += kg_dp;
+                    if (pc >= kg_row_pieces) {
+                        pc -= kg_row_pieces;
+                        ++r;
+                    }
+                }
             }
         }
     };
     auto slab_write = [&]() {
         if constexpr (KG) {
+            int r = kg_r, pc = kg_pc;
 #pragma unroll
             for (int i = 0; i < KG_MAX; ++i) {
-                const int idx = tid + i * NT;
-                if (idx < kg_pieces) {
-                    const int r = idx / (kg_groups * 2), pc = idx % (kg_groups * 2);
-                    *(uint4 *)(lds + (pc >> 1) * KG_GROUP + r * 32 + (r >> 3) * 32 + (pc & 1) * 16) = slab_v[i];
+                if (i * NT < kg_pieces) {
+                    if (r < RW)
+                        *(uint4 *)(lds + (pc >> 1) * KG_GROUP + r * 32 + (r >> 3) * 32 + (pc & 1) * 16) = slab_v[i];
+                    r += kg_dr;
+                    pc += kg_dp;
+                    if (pc >= kg_row_pieces) {
+                        pc -= kg_row_pieces;
+                        ++r;
+                    }
                 }
             }
         }
