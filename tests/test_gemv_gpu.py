@@ -187,8 +187,6 @@ def test_block_rotation_mode():
 @pytest.mark.parametrize("K", [64, 128, 192, 320, 448, 832, 1792, 2560, 5120, 6144, 8192, 16384])
 @pytest.mark.parametrize("N,bits,bits2", [(256, 4, 0), (2048, 4, 0), (512, 4, 4), (512, 2, 0)])
 def test_k_sweep_covers_every_loop_variant(K, N, bits, bits2):
-    if N == 2048 and K > 8192:
-        pytest.skip("covered by the narrower rows")
     w = make_weight(N, K, bits, 128, seed=K + N + bits, bits2=bits2, device=DEV)
     x = make_x(1, K, seed=11)
     y = _run(w, x).cpu()
