@@ -40,7 +40,8 @@ typedef enum flute_status {
 typedef enum flute_dtype {
     FLUTE_F16 = 0,
     FLUTE_BF16 = 1,
-    FLUTE_F32 = 2
+    FLUTE_F32 = 2,
+    FLUTE_U8 = 3           /* index blobs; only in flute_tensor records */
 } flute_dtype;
 
 /*
@@ -247,6 +248,46 @@ int flute_pick_split(int N, int K);
 /* LDS bytes one GEMV workgroup needs for this weight (0 when the weight is
  * refused); the host-side gates mirror it (flute_extended/__init__.py:643-665). */
 int64_t flute_gemv_lds_bytes(const flute_linear *w, int split);
+
+/*
+ * The argument checks of a binding, once.  Upstream's bindings check the tensors they are handed
+ * (dtype, rank, shape against K and the blob's byte count, contiguity, device) before they build
+ * a launch (src/bindings.cpp:230-546, src/kernel_gemv.cu:379-474); so must any binding of this
+ * library, and these two calls do it for them: the binding records what it knows about each
+ * tensor in a flute_tensor (no tensor type crosses the boundary) and gets back either the filled
+ * flute_linear and N, or FLUTE_ERR_INVALID with the message upstream's check would raise in
+ * flute_last_error().  "Absent" operands follow upstream's convention: an empty tensor
+ * (numel = 0); signs and awq are absent when `present` is 0.  Both bindings in this repository
+ * (flute_extended/_C.py over ctypes and csrc/torch_binding.cpp) call them, so the checks, their
+ * order and their messages exist in one place.  Pure host code: usable without a GPU.
+ */
+typedef struct flute_tensor {
+    const void *data;        /* address of element 0 (device memory for a GPU tensor) */
+    const char *dtype_name;  /* how the binding prints the dtype ("torch.float64"), or NULL */
+    int64_t numel;
+    int64_t size[4];         /* the first min(ndim, 4) sizes */
+    int32_t ndim;
+    int32_t dtype;           /* FLUTE_F16 / FLUTE_BF16 / FLUTE_F32 / FLUTE_U8, -1 for any other */
+    int32_t contiguous;
+    int32_t device;          /* ordinal of the GPU that holds it, -1 for host memory */
+    int32_t present;         /* 0: no such operand was passed (None) */
+    int32_t reserved;
+} flute_tensor;
+
+typedef struct flute_operands {
+    flute_tensor A, indices, lut, indices2, lut2, resB, resA, bias, signs, awq;
+    int64_t K;
+    int32_t b1, b2, group_size, rot_block;
+    int32_t max_rank;        /* largest residual rank the entry point accepts */
+    uint32_t gs_allowed;     /* bit i set: group size 2^i is accepted by the entry point */
+} flute_operands;
+
+/* A must be a contiguous 2-D float16/bfloat16 [M, K] with K % 64 == 0 (and M == 1 if need_m1). */
+flute_status flute_check_input(const char *who, const flute_tensor *A, int need_m1);
+/* Every check of one weight's operands; on success *out is ready for the launch entry points
+ * (data pointers as given: re-align misaligned blobs before the call) and *N_out is N. */
+flute_status flute_describe_linear(const char *who, const flute_operands *ops, flute_linear *out,
+                                   int64_t *N_out);
 
 /* Validate a weight descriptor exactly as the launchers do, without touching
  * the device.  mode: 0 = GEMV (accepts k_group = 128), 1 = GEMM (refuses it). */

@@ -49,15 +49,6 @@ const char *dtype_name(const Tensor &t) {
         default: return c10::toString(t.scalar_type());
     }
 }
-std::string shape_of(const Tensor &t) {
-    std::ostringstream s;
-    s << "(";
-    for (int64_t i = 0; i < t.dim(); ++i) s << (i ? ", " : "") << t.size(i);
-    if (t.dim() == 1) s << ",";
-    s << ")";
-    return s.str();
-}
-bool populated(const Tensor &t) { return t.defined() && t.numel() > 0; }
 
 void *stream_of(const Tensor &t) {
     return (void *)c10::hip::getCurrentHIPStream(t.device().index()).stream();
@@ -74,16 +65,43 @@ struct Shape2 {
     int64_t M, K;
 };
 
+// What the library's argument checks need to know about a tensor (flute_tensor): no tensor
+// type crosses the C ABI.  `name` keeps the printed dtype alive for the duration of the call.
+struct Record {
+    flute_tensor t = {};
+    std::string name;
+};
+void record(Record &r, const Tensor *t) {
+    if (t == nullptr || !t->defined()) {
+        r.t.present = 0;
+        return;
+    }
+    r.t.present = 1;
+    r.t.numel = t->numel();
+    r.t.ndim = (int32_t)t->dim();
+    for (int64_t i = 0; i < t->dim() && i < 4; ++i) r.t.size[i] = t->size(i);
+    switch (t->scalar_type()) {
+        case at::kHalf: r.t.dtype = FLUTE_F16; break;
+        case at::kBFloat16: r.t.dtype = FLUTE_BF16; break;
+        case at::kFloat: r.t.dtype = FLUTE_F32; break;
+        case at::kByte: r.t.dtype = FLUTE_U8; break;
+        default:
+            r.t.dtype = -1;
+            r.name = dtype_name(*t);
+            r.t.dtype_name = r.name.c_str();
+    }
+    r.t.contiguous = t->is_contiguous() ? 1 : 0;
+    r.t.device = t->is_cuda() ? (int32_t)t->device().index() : -1;
+    r.t.data = t->numel() ? t->data_ptr() : nullptr;
+}
+
+// The checks of the input matrix: flute_check_input (one copy for this binding and the ctypes
+// mirror).
 Shape2 check_2d_input(const char *who, const Tensor &A, bool need_m1) {
-    TORCH_CHECK(A.dim() == 2, who, ": A must be 2-D [M, K]");
-    TORCH_CHECK(is_act(A), who, ": A must be float16 or bfloat16 (got ", dtype_name(A), ")");
-    const int64_t M = A.size(0), K = A.size(1);
-    TORCH_CHECK(!need_m1 || M == 1, who, ": the decode GEMV serves M == 1 (got M=", M,
-                ") - route larger M through qgemm_dual_stream / qgemm_per_group_lut");
-    TORCH_CHECK(K % 64 == 0, who,
-                ": K must be a multiple of 64 (the idxN blob's 64-k tiles; got K=", K, ")");
-    TORCH_CHECK(A.is_contiguous(), who, ": A must be contiguous");
-    return {M, K};
+    Record r;
+    record(r, &A);
+    check_status(flute_check_input(who, &r.t, need_m1 ? 1 : 0));
+    return {A.size(0), A.size(1)};
 }
 
 struct Described {
@@ -92,146 +110,55 @@ struct Described {
     Tensor keep1, keep2;    // re-aligned blobs, alive until the launch is queued
 };
 
-bool gs_in(int64_t gs, const std::vector<int> &allowed) {
-    for (int g : allowed)
-        if (g == gs) return true;
-    return false;
-}
-std::string gs_list(const std::vector<int> &allowed) {
-    std::ostringstream s;
-    for (size_t i = 0; i < allowed.size(); ++i) s << (i ? "/" : "") << allowed[i];
-    return s.str();
+uint32_t gs_mask(const std::vector<int> &allowed) {
+    uint32_t m = 0;
+    for (int g : allowed) m |= 1u << (31 - __builtin_clz((unsigned)g));
+    return m;
 }
 
 const std::vector<int> kGsAll = {16, 32, 64, 128, 256, 512, 1024, 2048};
 const std::vector<int> kGsPlain = {64, 128, 256, 512, 1024, 2048};
 
-// The checks of one weight's tensors (flute_extended/_C.py::_describe, same order).
+// The checks of one weight's tensors: flute_describe_linear; this function records what it was
+// handed and re-aligns blobs that torch may hand over as views.
 Described describe(const char *who, const Tensor &A, int64_t K, const Tensor &indices,
                    const Tensor &lut, int64_t b1, const Tensor &indices2, const Tensor &lut2,
                    int64_t b2, const Tensor &resB, const Tensor &resA, const Tensor &bias,
                    int64_t gs, const c10::optional<Tensor> &signs, c10::optional<Tensor> awq,
                    int64_t rot_block, const std::vector<int> &gs_allowed, int64_t max_rank) {
-    TORCH_CHECK(b1 >= 1 && b1 <= 4, who, ": bitwidth must be 1, 2, 3 or 4 (got ", b1, ")");
-    TORCH_CHECK(b2 >= 0 && b2 <= 4, who,
-                ": bitwidth2 must be 0 (single stream) or 1..4 (got ", b2, ")");
-    TORCH_CHECK(gs_in(gs, gs_allowed), who, ": group_size must be one of ", gs_list(gs_allowed),
-                " (got ", gs, ")");
-    TORCH_CHECK(indices.scalar_type() == at::kByte, who, ": stream-1 indices must be uint8");
-    TORCH_CHECK(is_act(lut), who,
-                ": stream-1 lut must be float16 (or bfloat16 with bfloat16 activations)");
-    TORCH_CHECK(!(lut.scalar_type() == at::kBFloat16 && A.scalar_type() != at::kBFloat16), who,
-                ": a bfloat16 lut needs bfloat16 activations");
-    const int64_t row_bytes1 = (K * b1) / 8;
-    TORCH_CHECK(K != 0, who, ": K == 0 reaches the kernel path");
-    const int64_t N = indices.numel() / row_bytes1;
-    TORCH_CHECK(N > 0 && N * row_bytes1 == indices.numel(), who, ": stream-1 byte count ",
-                indices.numel(), " is not N*(K*", b1, "/8) for any N (K = ", K, ")");
-    TORCH_CHECK(N % 128 == 0, who, ": idxN layout requires N % 128 == 0 (got N = ", N, ")");
-    const int64_t rows = (N + gs - 1) / gs;
-    TORCH_CHECK(lut.dim() == 2 && lut.size(0) == rows && lut.size(1) == (1 << b1), who,
-                ": stream-1 lut must be [ceil(N/group_size), 2^bitwidth] = [", rows, ", ",
-                (1 << b1), "] (got ", shape_of(lut), ")");
-    TORCH_CHECK(indices.is_contiguous() && lut.is_contiguous(), who,
-                ": stream-1 indices and lut must be contiguous");
-    const bool has_s2 = b2 > 0;
-    if (has_s2) {
-        TORCH_CHECK(indices2.scalar_type() == at::kByte, who, ": stream-2 indices must be uint8");
-        TORCH_CHECK(lut2.scalar_type() == lut.scalar_type(), who,
-                    ": stream-2 lut must have the dtype of stream 1 (", dtype_name(lut), ")");
-        TORCH_CHECK(indices2.numel() == N * ((K * b2) / 8), who, ": stream-2 byte count ",
-                    indices2.numel(), " != N*K*", b2, "/8 = ", N * ((K * b2) / 8));
-        TORCH_CHECK(lut2.dim() == 2 && lut2.size(0) == rows && lut2.size(1) == (1 << b2), who,
-                    ": stream-2 lut must be [ceil(N/group_size), 2^bitwidth2] = [", rows, ", ",
-                    (1 << b2), "] (got ", shape_of(lut2), ")");
-        TORCH_CHECK(indices2.is_contiguous() && lut2.is_contiguous(), who,
-                    ": stream-2 indices/lut must be contiguous");
-    }
-    const bool has_res = populated(resB);
-    TORCH_CHECK(has_res == populated(resA), who,
-                ": resB and resA must be supplied together (both empty or both populated)");
-    int64_t R = 0;
-    if (has_res) {
-        TORCH_CHECK(resB.scalar_type() == A.scalar_type() && resA.scalar_type() == A.scalar_type(),
-                    who, ": resB/resA must have the activation dtype ", dtype_name(A));
-        TORCH_CHECK(resB.dim() == 2 && resA.dim() == 2, who,
-                    ": resB must be (R, K) and resA (N, R)");
-        R = resB.size(0);
-        TORCH_CHECK(R >= 1 && R <= max_rank, who, ": residual rank must be 1..", max_rank,
-                    " (got R=", R, ")");
-        TORCH_CHECK(resB.size(1) == K && resA.size(0) == N && resA.size(1) == R, who,
-                    ": residual shape mismatch: resB ", shape_of(resB), ", resA ", shape_of(resA),
-                    " for N=", N, ", K=", K);
-        TORCH_CHECK(resB.is_contiguous() && resA.is_contiguous(), who,
-                    ": resB/resA must be contiguous");
-    }
-    const bool has_bias = populated(bias);
-    if (has_bias)
-        TORCH_CHECK(bias.scalar_type() == A.scalar_type() && bias.dim() == 1 && bias.size(0) == N &&
-                        bias.is_contiguous(),
-                    who, ": bias must be a contiguous (N,) ", dtype_name(A), " tensor (N=", N, ")");
-    const bool has_signs = signs.has_value() && signs->defined();
-    if (has_signs)
-        TORCH_CHECK(signs->scalar_type() == at::kFloat && signs->dim() == 1 &&
-                        signs->numel() == K && signs->is_contiguous(),
-                    who, ": signs must be a contiguous (K,) float32 vector (K=", K, ")");
-    bool has_awq = awq.has_value() && populated(*awq);
-    if (has_awq) {
-        TORCH_CHECK(has_signs, who, ": awq scale without rotation signs");
-        TORCH_CHECK(awq->scalar_type() == at::kFloat && awq->dim() == 1 && awq->numel() == K &&
-                        awq->is_contiguous(),
-                    who, ": awq scale must be a contiguous (K,) float32 vector (K=", K, ")");
-    }
-
-    // ---- device --------------------------------------------------------------------
-    std::vector<const Tensor *> tensors = {&A, &indices, &lut};
-    if (has_s2) {
-        tensors.push_back(&indices2);
-        tensors.push_back(&lut2);
-    }
-    if (has_res) {
-        tensors.push_back(&resB);
-        tensors.push_back(&resA);
-    }
-    if (has_bias) tensors.push_back(&bias);
-    if (has_signs) tensors.push_back(&*signs);
-    if (has_awq) tensors.push_back(&*awq);
-    for (const Tensor *t : tensors) {
-        TORCH_CHECK(t->is_cuda(), who, ": all tensors must be CUDA (HIP) tensors");
-        TORCH_CHECK(t->device() == A.device(), who, ": all tensors must live on A's device ",
-                    A.device().str());
-    }
-
     Described d;
-    d.N = N;
-    d.keep1 = aligned16(indices);
-    flute_linear &w = d.w;
-    w = flute_linear{};
-    w.q1 = d.keep1.data_ptr();
-    w.lut1 = lut.data_ptr();
-    w.q1_bytes = indices.numel();
-    if (has_s2) {
-        d.keep2 = aligned16(indices2);
-        w.q2 = d.keep2.data_ptr();
-        w.lut2 = lut2.data_ptr();
-        w.q2_bytes = indices2.numel();
-    }
-    if (has_res) {
-        w.resB = resB.data_ptr();
-        w.resA = resA.data_ptr();
-    }
-    if (has_bias) w.bias = bias.data_ptr();
-    if (has_signs) w.signs = (const float *)signs->data_ptr();
-    if (has_awq) w.awq = (const float *)awq->data_ptr();
-    w.lut_rows = (int)rows;
-    w.N = (int)N;
-    w.K = (int)K;
-    w.R = (int)R;
-    w.b1 = (int)b1;
-    w.b2 = (int)b2;
-    w.group_size = (int)gs;
-    w.lut_dtype = act_code(lut);
-    w.rot_block = (int)rot_block;
+    d.keep1 = (indices.defined() && indices.is_cuda()) ? aligned16(indices) : indices;
+    d.keep2 = (b2 > 0 && indices2.defined() && indices2.is_cuda()) ? aligned16(indices2) : indices2;
+    Record rA, rI, rL, rI2, rL2, rRB, rRA, rBias, rS, rAwq;
+    record(rA, &A);
+    record(rI, &d.keep1);
+    record(rL, &lut);
+    record(rI2, &d.keep2);
+    record(rL2, &lut2);
+    record(rRB, &resB);
+    record(rRA, &resA);
+    record(rBias, &bias);
+    record(rS, signs.has_value() ? &*signs : nullptr);
+    record(rAwq, awq.has_value() ? &*awq : nullptr);
+    flute_operands ops = {};
+    ops.A = rA.t;
+    ops.indices = rI.t;
+    ops.lut = rL.t;
+    ops.indices2 = rI2.t;
+    ops.lut2 = rL2.t;
+    ops.resB = rRB.t;
+    ops.resA = rRA.t;
+    ops.bias = rBias.t;
+    ops.signs = rS.t;
+    ops.awq = rAwq.t;
+    ops.K = K;
+    ops.b1 = (int32_t)b1;
+    ops.b2 = (int32_t)b2;
+    ops.group_size = (gs >= INT32_MIN && gs <= INT32_MAX) ? (int32_t)gs : -1;
+    ops.rot_block = (int32_t)rot_block;
+    ops.max_rank = (int32_t)max_rank;
+    ops.gs_allowed = gs_mask(gs_allowed);
+    check_status(flute_describe_linear(who, &ops, &d.w, &d.N));
     return d;
 }
 

@@ -78,145 +78,101 @@ def _aligned16(t: torch.Tensor) -> torch.Tensor:
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
+_DTYPE_CODE = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32,
+               torch.uint8: _lib.U8}
+_DTYPE_NAME = {}
+
+
+def _record(rec: "_lib.FluteTensor", t: Optional[torch.Tensor]) -> None:
+    """Fill one flute_tensor record from a tensor (None: the operand was not passed)."""
+    if t is None:
+        rec.present = 0
+        return
+    rec.present = 1
+    n = t.numel()
+    if n == 0:
+        # upstream's "absent operand": only the emptiness is looked at, unless the entry's own
+        # arguments (a second bit width) say the operand is needed, and then it fails on its size
+        rec.ndim = t.dim()
+        if rec.ndim > 1:
+            for i, v in enumerate(t.shape[:4]):
+                rec.size[i] = v
+        rec.dtype = _DTYPE_CODE.get(t.dtype, -1)
+        rec.contiguous = 1
+        rec.device = -1
+        return
+    rec.numel = n
+    rec.ndim = t.dim()
+    for i, n in enumerate(t.shape[:4]):
+        rec.size[i] = n
+    code = _DTYPE_CODE.get(t.dtype, -1)
+    rec.dtype = code
+    if code < 0:
+        name = _DTYPE_NAME.get(t.dtype)
+        if name is None:
+            name = _DTYPE_NAME[t.dtype] = str(t.dtype).encode()
+        rec.dtype_name = name
+    rec.contiguous = 1 if t.is_contiguous() else 0
+    rec.device = (t.device.index if t.device.index is not None else torch.cuda.current_device()) \
+        if t.is_cuda else -1
+    rec.data = t.data_ptr()
+
+
 def _check_2d_input(who: str, A: torch.Tensor, need_m1: bool) -> tuple:
-    if A.dim() != 2:
-        _fail(f"{who}: A must be 2-D [M, K]")
-    if A.dtype not in _ACT:
-        _fail(f"{who}: A must be float16 or bfloat16 (got {A.dtype})")
-    M, K = int(A.shape[0]), int(A.shape[1])
-    if need_m1 and M != 1:
-        _fail(f"{who}: the decode GEMV serves M == 1 (got M={M}) - route larger M through "
-              "qgemm_dual_stream / qgemm_per_group_lut")
-    if K % 64 != 0:
-        _fail(f"{who}: K must be a multiple of 64 (the idxN blob's 64-k tiles; got K={K})")
-    if not A.is_contiguous():
-        _fail(f"{who}: A must be contiguous")
-    return M, K
+    """The checks of the input matrix (flute_check_input in the library: one copy for this mirror
+    and the compiled binding)."""
+    rec = _lib.FluteTensor()
+    _record(rec, A)
+    if lib.flute_check_input(who.encode(), ctypes.byref(rec), 1 if need_m1 else 0) != _lib.FLUTE_OK:
+        _fail(_lib.last_error())
+    return int(A.shape[0]), int(A.shape[1])
+
+
+def _gs_mask(sizes: Sequence[int]) -> int:
+    mask = 0
+    for g in sizes:
+        mask |= 1 << (int(g).bit_length() - 1)
+    return mask
+
+
+_GS_MASKS = {}
 
 
 def _describe(who: str, A: torch.Tensor, K: int, indices, lut, bitwidth, indices2, lut2,
               bitwidth2, resB, resA, bias, group_size, signs=None, awq=None,
               rot_block: int = 0, gs_allowed: Sequence[int] = _GS_ALL,
               max_rank: int = 256):
-    """Validate one weight's tensors and return (FluteLinear, N, keepalive)."""
-    b1, b2 = int(bitwidth), int(bitwidth2)
-    if not 1 <= b1 <= 4:
-        _fail(f"{who}: bitwidth must be 1, 2, 3 or 4 (got {b1})")
-    if not 0 <= b2 <= 4:
-        _fail(f"{who}: bitwidth2 must be 0 (single stream) or 1..4 (got {b2})")
-    gs = int(group_size)
-    if gs not in gs_allowed:
-        _fail(f"{who}: group_size must be one of {'/'.join(map(str, gs_allowed))} (got {gs})")
-    if indices.dtype != torch.uint8:
-        _fail(f"{who}: stream-1 indices must be uint8")
-    if lut.dtype not in _ACT:
-        _fail(f"{who}: stream-1 lut must be float16 (or bfloat16 with bfloat16 activations)")
-    if lut.dtype == torch.bfloat16 and A.dtype != torch.bfloat16:
-        _fail(f"{who}: a bfloat16 lut needs bfloat16 activations")
-    row_bytes1 = (K * b1) // 8
-    if K == 0:
-        _fail(f"{who}: K == 0 reaches the kernel path")
-    N = indices.numel() // row_bytes1
-    if N <= 0 or N * row_bytes1 != indices.numel():
-        _fail(f"{who}: stream-1 byte count {indices.numel()} is not N*(K*{b1}/8) for any N "
-              f"(K = {K})")
-    if N % 128 != 0:
-        _fail(f"{who}: idxN layout requires N % 128 == 0 (got N = {N})")
-    rows = (N + gs - 1) // gs
-    if lut.dim() != 2 or lut.shape[0] != rows or lut.shape[1] != (1 << b1):
-        _fail(f"{who}: stream-1 lut must be [ceil(N/group_size), 2^bitwidth] = "
-              f"[{rows}, {1 << b1}] (got {tuple(lut.shape)})")
-    if not (indices.is_contiguous() and lut.is_contiguous()):
-        _fail(f"{who}: stream-1 indices and lut must be contiguous")
-    has_s2 = b2 > 0
-    if has_s2:
-        if indices2.dtype != torch.uint8:
-            _fail(f"{who}: stream-2 indices must be uint8")
-        if lut2.dtype != lut.dtype:
-            _fail(f"{who}: stream-2 lut must have the dtype of stream 1 ({lut.dtype})")
-        if indices2.numel() != N * ((K * b2) // 8):
-            _fail(f"{who}: stream-2 byte count {indices2.numel()} != N*K*{b2}/8 = "
-                  f"{N * ((K * b2) // 8)}")
-        if lut2.dim() != 2 or lut2.shape[0] != rows or lut2.shape[1] != (1 << b2):
-            _fail(f"{who}: stream-2 lut must be [ceil(N/group_size), 2^bitwidth2] = "
-                  f"[{rows}, {1 << b2}] (got {tuple(lut2.shape)})")
-        if not (indices2.is_contiguous() and lut2.is_contiguous()):
-            _fail(f"{who}: stream-2 indices/lut must be contiguous")
-    has_res = resB is not None and resB.numel() > 0
-    if has_res != (resA is not None and resA.numel() > 0):
-        _fail(f"{who}: resB and resA must be supplied together (both empty or both populated)")
-    R = 0
-    if has_res:
-        if resB.dtype != A.dtype or resA.dtype != A.dtype:
-            _fail(f"{who}: resB/resA must have the activation dtype {A.dtype}")
-        if resB.dim() != 2 or resA.dim() != 2:
-            _fail(f"{who}: resB must be (R, K) and resA (N, R)")
-        R = int(resB.shape[0])
-        if not 1 <= R <= max_rank:
-            _fail(f"{who}: residual rank must be 1..{max_rank} (got R={R})")
-        if resB.shape[1] != K or resA.shape[0] != N or resA.shape[1] != R:
-            _fail(f"{who}: residual shape mismatch: resB {tuple(resB.shape)}, resA "
-                  f"{tuple(resA.shape)} for N={N}, K={K}")
-        if not (resB.is_contiguous() and resA.is_contiguous()):
-            _fail(f"{who}: resB/resA must be contiguous")
-    has_bias = bias is not None and bias.numel() > 0
-    if has_bias:
-        if bias.dtype != A.dtype or bias.dim() != 1 or bias.shape[0] != N \
-                or not bias.is_contiguous():
-            _fail(f"{who}: bias must be a contiguous (N,) {A.dtype} tensor (N={N})")
-    if signs is not None:
-        if signs.dtype != torch.float32 or signs.dim() != 1 or signs.numel() != K \
-                or not signs.is_contiguous():
-            _fail(f"{who}: signs must be a contiguous (K,) float32 vector (K={K})")
-    if awq is not None and awq.numel() > 0:
-        if signs is None:
-            _fail(f"{who}: awq scale without rotation signs")
-        if awq.dtype != torch.float32 or awq.dim() != 1 or awq.numel() != K \
-                or not awq.is_contiguous():
-            _fail(f"{who}: awq scale must be a contiguous (K,) float32 vector (K={K})")
-    else:
-        awq = None
-
-    # ---- device ----------------------------------------------------------------
-    tensors = [A, indices, lut]
-    if has_s2:
-        tensors += [indices2, lut2]
-    if has_res:
-        tensors += [resB, resA]
-    if has_bias:
-        tensors.append(bias)
-    if signs is not None:
-        tensors.append(signs)
-    if awq is not None:
-        tensors.append(awq)
-    for t in tensors:
-        if not t.is_cuda:
-            _fail(f"{who}: all tensors must be CUDA (HIP) tensors")
-        if t.device != A.device:
-            _fail(f"{who}: all tensors must live on A's device {A.device}")
-
-    indices = _aligned16(indices)
-    if has_s2:
+    """Validate one weight's tensors and return (FluteLinear, N, keepalive).  The checks
+    themselves are flute_describe_linear's: this function only records what it was given."""
+    indices = _aligned16(indices) if indices.is_cuda else indices
+    if int(bitwidth2) > 0 and indices2 is not None and indices2.is_cuda:
         indices2 = _aligned16(indices2)
+    ops = _lib.FluteOperands()
+    _record(ops.A, A)
+    _record(ops.indices, indices)
+    _record(ops.lut, lut)
+    _record(ops.indices2, indices2)
+    _record(ops.lut2, lut2)
+    _record(ops.resB, resB)
+    _record(ops.resA, resA)
+    _record(ops.bias, bias)
+    _record(ops.signs, signs)
+    _record(ops.awq, awq)
+    ops.K, ops.b1, ops.b2 = int(K), int(bitwidth), int(bitwidth2)
+    gs = int(group_size)
+    ops.group_size = gs if -2 ** 31 <= gs < 2 ** 31 else -1
+    ops.rot_block, ops.max_rank = int(rot_block), int(max_rank)
+    key = tuple(gs_allowed)
+    mask = _GS_MASKS.get(key)
+    if mask is None:
+        mask = _GS_MASKS[key] = _gs_mask(key)
+    ops.gs_allowed = mask
     w = FluteLinear()
-    w.q1, w.lut1 = indices.data_ptr(), lut.data_ptr()
-    w.q1_bytes = indices.numel()
-    if has_s2:
-        w.q2, w.lut2 = indices2.data_ptr(), lut2.data_ptr()
-        w.q2_bytes = indices2.numel()
-    if has_res:
-        w.resB, w.resA = resB.data_ptr(), resA.data_ptr()
-    if has_bias:
-        w.bias = bias.data_ptr()
-    if signs is not None:
-        w.signs = signs.data_ptr()
-    if awq is not None:
-        w.awq = awq.data_ptr()
-    w.lut_rows, w.N, w.K, w.R = rows, N, K, R
-    w.b1, w.b2, w.group_size = b1, b2, gs
-    w.lut_dtype = _ACT[lut.dtype]
-    w.rot_block = int(rot_block)
-    return w, N, (indices, indices2)
+    n = ctypes.c_int64(0)
+    if lib.flute_describe_linear(who.encode(), ctypes.byref(ops), ctypes.byref(w),
+                                 ctypes.byref(n)) != _lib.FLUTE_OK:
+        _fail(_lib.last_error())
+    return w, int(n.value), (indices, indices2)
 
 
 def _gemv(who, A, indices, lut, bitwidth, indices2, lut2, bitwidth2, resB, resA, bias,

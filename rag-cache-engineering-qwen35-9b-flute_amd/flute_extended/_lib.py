@@ -18,7 +18,7 @@ FLUTE_ERR_UNSUPPORTED = 2
 FLUTE_ERR_HIP = 3
 FLUTE_ERR_NOMEM = 4
 
-F16, BF16, F32 = 0, 1, 2
+F16, BF16, F32, U8 = 0, 1, 2, 3
 
 
 class FluteLinear(ctypes.Structure):
@@ -48,6 +48,36 @@ class FluteLinear(ctypes.Structure):
     ]
 
 
+class FluteTensor(ctypes.Structure):
+    """struct flute_tensor: what a binding knows about one tensor."""
+    _fields_ = [
+        ("data", ctypes.c_void_p),
+        ("dtype_name", ctypes.c_char_p),
+        ("numel", ctypes.c_int64),
+        ("size", ctypes.c_int64 * 4),
+        ("ndim", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("contiguous", ctypes.c_int32),
+        ("device", ctypes.c_int32),
+        ("present", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+class FluteOperands(ctypes.Structure):
+    """struct flute_operands: the operands of one weight as an entry point received them."""
+    _fields_ = [(n, FluteTensor) for n in
+                ("A", "indices", "lut", "indices2", "lut2", "resB", "resA", "bias", "signs", "awq")] + [
+        ("K", ctypes.c_int64),
+        ("b1", ctypes.c_int32),
+        ("b2", ctypes.c_int32),
+        ("group_size", ctypes.c_int32),
+        ("rot_block", ctypes.c_int32),
+        ("max_rank", ctypes.c_int32),
+        ("gs_allowed", ctypes.c_uint32),
+    ]
+
+
 # every symbol include/flute_hip.h declares: (restype, argtypes)
 _P = ctypes.c_void_p
 _LP = ctypes.POINTER(FluteLinear)
@@ -56,6 +86,9 @@ SYMBOLS = {
     "flute_abi_version": (_I, []),
     "flute_last_error": (ctypes.c_char_p, []),
     "flute_target_arch": (ctypes.c_char_p, []),
+    "flute_check_input": (_I, [ctypes.c_char_p, ctypes.POINTER(FluteTensor), _I]),
+    "flute_describe_linear": (_I, [ctypes.c_char_p, ctypes.POINTER(FluteOperands), _LP,
+                                   ctypes.POINTER(ctypes.c_int64)]),
     "flute_gemv": (_I, [_LP, _P, _P, _I, _I, _P]),
     "flute_gemv_noalloc": (_I, [_LP, _P, _P, _I, _I, _P]),
     "flute_gemv_mlp": (_I, [_LP, _LP, _P, _P, _I, _I, _P]),

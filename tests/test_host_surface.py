@@ -221,6 +221,79 @@ def test_tensor_level_refusals_raise_runtimeerror():
         fx.qgemm_gemv_stream(x, w["blob"], w["lut"], 4, 32)         # plain entry: gs >= 64 only
 
 
+def _rec(rec, shape, dtype, device=0, data=4096, present=1, name=None, contiguous=1):
+    rec.present, rec.ndim, rec.dtype, rec.device, rec.contiguous = present, len(shape), dtype, device, contiguous
+    n = 1
+    for i, v in enumerate(shape):
+        rec.size[i] = v
+        n *= v
+    rec.numel = n if shape else 0
+    rec.data = data if n else None
+    if name:
+        rec.dtype_name = name
+
+
+def _operands(N=256, K=128, b1=4, gs=128, **over):
+    ops = _lib.FluteOperands()
+    _rec(ops.A, (1, K), _lib.F16)
+    _rec(ops.indices, (N * K * b1 // 8,), _lib.U8)
+    _rec(ops.lut, ((N + gs - 1) // gs, 1 << b1), _lib.F16)
+    for name in ("indices2", "lut2", "resB", "resA", "bias"):
+        _rec(getattr(ops, name), (0,), _lib.F16)
+    ops.signs.present = ops.awq.present = 0
+    ops.K, ops.b1, ops.b2, ops.group_size, ops.max_rank = K, b1, 0, gs, 256
+    ops.gs_allowed = sum(1 << i for i in range(4, 12))
+    for k, v in over.items():
+        v(ops) if callable(v) else setattr(ops, k, v)
+    return ops
+
+
+def test_the_library_s_own_argument_checks_fill_the_descriptor():
+    """flute_describe_linear from plain records, no tensor library involved: the descriptor it
+    returns, and one refusal of each kind with upstream's message."""
+    def run(ops):
+        w, n = _lib.FluteLinear(), ctypes.c_int64(0)
+        st = _lib.lib.flute_describe_linear(b"entry", ctypes.byref(ops), ctypes.byref(w), ctypes.byref(n))
+        return st, w, n.value, _lib.last_error()
+    st, w, n, _ = run(_operands())
+    assert st == _lib.FLUTE_OK and n == 256
+    assert (w.N, w.K, w.b1, w.b2, w.R, w.group_size, w.lut_rows, w.q1_bytes) == (256, 128, 4, 0, 0, 128, 2, 16384)
+    assert w.q1 == 4096 and w.lut1 == 4096 and not w.q2 and not w.resA and not w.signs and w.k_group == 0
+    assert _lib.lib.flute_validate(ctypes.byref(w), 0) == _lib.FLUTE_OK
+    cases = [
+        (dict(b1=5), "entry: bitwidth must be 1, 2, 3 or 4 (got 5)"),
+        (dict(group_size=48), "entry: group_size must be one of 16/32/64/128/256/512/1024/2048 (got 48)"),
+        (dict(gs_allowed=sum(1 << i for i in range(6, 12)), group_size=32),
+         "entry: group_size must be one of 64/128/256/512/1024/2048 (got 32)"),
+        (dict(x=lambda o: _rec(o.indices, (16377,), _lib.U8)),
+         "entry: stream-1 byte count 16377 is not N*(K*4/8) for any N (K = 128)"),
+        (dict(x=lambda o: _rec(o.lut, (2, 8), _lib.F16)),
+         "entry: stream-1 lut must be [ceil(N/group_size), 2^bitwidth] = [2, 16] (got (2, 8))"),
+        (dict(x=lambda o: _rec(o.lut, (2, 16), _lib.BF16)), "entry: a bfloat16 lut needs bfloat16 activations"),
+        (dict(x=lambda o: _rec(o.resB, (4, 128), _lib.F16)),
+         "entry: resB and resA must be supplied together (both empty or both populated)"),
+        (dict(x=lambda o: _rec(o.bias, (7,), _lib.F16)),
+         "entry: bias must be a contiguous (N,) torch.float16 tensor (N=256)"),
+        (dict(x=lambda o: _rec(o.signs, (64,), _lib.F32)),
+         "entry: signs must be a contiguous (K,) float32 vector (K=128)"),
+        (dict(x=lambda o: _rec(o.awq, (128,), _lib.F32)), "entry: awq scale without rotation signs"),
+        (dict(x=lambda o: _rec(o.lut, (2, 16), _lib.F16, device=-1)), "entry: all tensors must be CUDA (HIP) tensors"),
+        (dict(x=lambda o: _rec(o.lut, (2, 16), _lib.F16, device=1)),
+         "entry: all tensors must live on A's device cuda:0"),
+    ]
+    for over, msg in cases:
+        st, _, _, err = run(_operands(**over))
+        assert st == _lib.FLUTE_ERR_INVALID and err == msg, (over, err)
+    a = _lib.FluteTensor()
+    _rec(a, (1, 128), -1, name=b"torch.float64")
+    assert _lib.lib.flute_check_input(b"entry", ctypes.byref(a), 1) == _lib.FLUTE_ERR_INVALID
+    assert _lib.last_error() == "entry: A must be float16 or bfloat16 (got torch.float64)"
+    _rec(a, (3, 128), _lib.BF16)
+    assert _lib.lib.flute_check_input(b"entry", ctypes.byref(a), 0) == _lib.FLUTE_OK
+    assert _lib.lib.flute_check_input(b"entry", ctypes.byref(a), 1) == _lib.FLUTE_ERR_INVALID
+    assert "M == 1 (got M=3)" in _lib.last_error()
+
+
 def _first_line(fn):
     with pytest.raises(RuntimeError) as err:
         fn()
@@ -229,8 +302,9 @@ def _first_line(fn):
 
 @pytest.mark.skipif(_C.native is None, reason="the compiled binding is not built or switched off")
 def test_compiled_binding_refuses_with_the_python_binding_s_words():
-    """csrc/torch_binding.cpp restates the checks of flute_extended/_C.py (upstream: the
-    TORCH_CHECKs of src/kernel_gemv.cu:338-454): same order, same first line."""
+    """csrc/torch_binding.cpp and flute_extended/_C.py hand their tensors to the same checks in
+    the library (upstream: the TORCH_CHECKs of src/kernel_gemv.cu:338-454): same order, same
+    first line, whichever binding recorded the tensors."""
     x, w = _cpu_args()
     e8 = torch.empty(0, dtype=torch.uint8)
     e16 = torch.empty(0, dtype=torch.float16)
