@@ -122,6 +122,59 @@ def test_fused_rotation(block):
     assert rel_l2(y, exact(xr.half(), dense(idx, lut)).half()) <= TOL
 
 
+@pytest.mark.parametrize("rot", [False, True])
+def test_residual_bias_and_rotation_through_the_descriptor(rot):
+    """The low-rank residual, the bias and the rotation do not depend on how the LUT is grouped:
+    a descriptor that carries all of them must give x_rot . W^T + (x_rot . resB^T) . resA^T + bias."""
+    N, K, R = 512, 2048, 8
+    idx, lut, blob = make_kgroup(N, K, 37)
+    g = torch.Generator().manual_seed(38)
+    resB = (torch.randn(R, K, generator=g) * 0.05).half()
+    resA = (torch.randn(N, R, generator=g) * 0.05).half()
+    bias = (torch.randn(N, generator=g) * 0.1).half()
+    x = make_x(1, K, seed=17)
+    signs = O.rotation_signs(K, 5)
+    xr = O.fht_reference(x, signs).half() if rot else x
+    want = exact(xr, dense(idx, lut), bias) + (xr.double() @ resB.double().t()) @ resA.double().t()
+    xd, blob_d, lut_d = x.to(DEV), blob.to(DEV), lut.to(DEV)
+    keep = [resB.to(DEV), resA.to(DEV), bias.to(DEV), signs.to(DEV)]
+    w, _, keep2 = _C._describe_kgroup("test", xd, K, blob_d, lut_d, bias=keep[2],
+                                      signs=keep[3] if rot else None)
+    w.resB, w.resA, w.R = keep[0].data_ptr(), keep[1].data_ptr(), R
+    out = torch.empty(1, N, dtype=torch.float16, device=DEV)
+    _lib.check(_lib.lib.flute_gemv(ctypes.byref(w), xd.data_ptr(), out.data_ptr(), _lib.F16, 0,
+                                   torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert rel_l2(out.cpu(), want.half()) <= TOL
+
+
+def test_noalloc_entry_replays_from_a_graph():
+    """The allocation-free entry with a K split (tickets and partial sums in its fixed array),
+    captured once and replayed: every replay must equal the eager result."""
+    N, K, split = 256, 4096, 2
+    idx, lut, blob = make_kgroup(N, K, 41)
+    x = make_x(1, K, seed=18).to(DEV)
+    blob_d, lut_d = blob.to(DEV), lut.to(DEV)
+    want = fx.qgemm_gemv_kgroup(x, blob_d, lut_d, split=split)
+    w, _, keep = _C._describe_kgroup("test", x, K, blob_d, lut_d)
+    out = torch.zeros_like(want)
+
+    def call():
+        _lib.check(_lib.lib.flute_gemv_noalloc(ctypes.byref(w), x.data_ptr(), out.data_ptr(), _lib.F16,
+                                               split, torch.cuda.current_stream().cuda_stream))
+    call()                                             # resolves the array's address outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+
+
 def test_noalloc_entry_matches():
     N, K, split = 512, 4096, 4
     idx, lut, blob = make_kgroup(N, K, 29)
