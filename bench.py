@@ -304,23 +304,31 @@ def _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, down, keep_down,
     del two, keep2
     # LUT grouped along K: one row of 16 values per (output row, 128-wide K group), [N, K/128, 16]
     # (a form no upstream artifact has; bytes = indices + that LUT = 37,748,736 at 4096 -> 12288)
-    kluts = [(torch.randn(I, H // 128, 16, device=dev, generator=gen) * 0.02).sort(dim=2).values
-             .to(torch.float16).contiguous() for _ in gate]
-    kds = []
-    for g_, kl in zip(gate, kluts):
-        d = _copy_desc(_lib, ctypes, g_)
-        d.lut1, d.lut_rows, d.k_group, d.lut_dtype = kl.data_ptr(), I * (H // 128), 128, _lib.F16
-        kds.append(d)
+    def k_grouped(name, descs, blobs, N, K, xin):
+        kluts = [(torch.randn(N, K // 128, 16, device=dev, generator=gen) * 0.02).sort(dim=2).values
+                 .to(torch.float16).contiguous() for _ in descs]
+        kds = []
+        for g_, kl in zip(descs, kluts):
+            d = _copy_desc(_lib, ctypes, g_)
+            d.lut1, d.lut_rows, d.k_group, d.lut_dtype = kl.data_ptr(), N * (K // 128), 128, _lib.F16
+            kds.append(d)
 
-    def krows(t):
-        per = (H // 64) * 1024 * 4
-        idx = torch.from_numpy(O.unpack_idxn(keep[0][0][t * per:(t + 1) * per].cpu().numpy(), 128, H, 4)).long()
-        lk = kluts[0][t * 128:(t + 1) * 128].cpu().double()           # [128, K/128, 16]
-        grp = (torch.arange(H) // 128)[None, :].expand(128, H)
-        return lk[torch.arange(128)[:, None].expand(128, H), grp, idx]
-    out["gemv_4096x12288_lut_grouped_along_k"] = gv.run(
-        "k_grouped_lut", kds, keep, I, H, x, rows_of=krows, wbytes=I * H // 2 + I * (H // 128) * 32)
-    del kds, kluts
+        def krows(t):
+            per = (K // 64) * 1024 * 4
+            idx = torch.from_numpy(O.unpack_idxn(blobs[0][0][t * per:(t + 1) * per].cpu().numpy(), 128, K, 4)).long()
+            lk = kluts[0][t * 128:(t + 1) * 128].cpu().double()           # [128, K/128, 16]
+            grp = (torch.arange(K) // 128)[None, :].expand(128, K)
+            return lk[torch.arange(128)[:, None].expand(128, K), grp, idx]
+        res = gv.run(name, kds, blobs, N, K, xin, rows_of=krows, wbytes=N * K // 2 + N * (K // 128) * 32)
+        res["bytes_index_plus_lut"] = N * K // 2 + N * (K // 128) * 32
+        return res
+    out["gemv_4096x12288_lut_grouped_along_k"] = k_grouped("k_grouped_lut", gate, keep, I, H, x)
+    out["gemv_12288x4096_lut_grouped_along_k"] = k_grouped(
+        "k_grouped_lut_down", down, keep_down, H, I, torch.randn(1, I, device=dev, generator=gen).to(x.dtype))
+    ws0 = [_weights(torch, H, H, gen, dev, torch.float16) for _ in range(count0)]
+    out["gemv_config0_4096x4096_fp16_lut_grouped_along_k"] = k_grouped(
+        "config0_k_grouped_lut", [_desc(_lib, b, l, H, H) for b, l in ws0], ws0, H, H, x16)
+    del ws0
     # fused rotations
     signs = (torch.randint(0, 2, (H,), device=dev, generator=gen).float() * 2 - 1).contiguous()
     signs_d = (torch.randint(0, 2, (I,), device=dev, generator=gen).float() * 2 - 1).contiguous()
