@@ -180,7 +180,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
     if (k_group) {
         // Only the lean kernel serves this form: four or eight wavefronts, each with an even
         // number (two at least) of loads of 32 / rw tiles.  The workgroup stages its LUT rows in
-        // LDS, 32 bytes per (row, K group), at most kKGroupPieces 16-byte pieces per thread, whole
+        // LDS, 64 bytes per (row, K group), at most kKGroupPieces 16-byte pieces per thread, whole
         // K groups per split.  The shape chosen above is kept where it fits; else wider slices or
         // another wavefront count; else, where the library chooses the split, a larger one.
         auto ok = [&](int sp, int rw_, int wv) {
@@ -306,7 +306,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
             if (es < entry_bytes_log2(gs.bits)) es = entry_bytes_log2(gs.bits);
             if (k_group) es = 7;            // (no table: the lean kernel's LUT rows, sized below)
             gs.es = es;
-            const size_t tb = k_group ? (size_t)(kc / 128) * (rw * 32 + (rw / 8) * 32)
+            const size_t tb = k_group ? (size_t)(kc / 128) * (rw * 64 + (rw / 8) * 64)
                                       : ((size_t)1 << (entries_log2(gs.bits) + es)) << ngrp_log2;
             if (tb > tab_bytes) tab_bytes = tb;
         }

@@ -207,10 +207,12 @@ constexpr int kKGroupPieces = 8;
 // KG: the LUT is grouped along K instead of along N: one row of sixteen values per (output row,
 // 128-wide K group), W[n, k] = LUT[n][k / 128][idx[n, k]] (a variant no upstream artifact has;
 // single weight, one 4-bit stream).  No pair table then (it would be 1 KB per 128 weights): the
-// workgroup stages the LUT rows of its row slice and K range in LDS, group-major with the rows
-// of a group 32 bytes apart, and a weight is one 16-bit read at (code * 2) in its row.  A row is
-// eight dwords on eight different banks and equal dwords are broadcast, so the lanes of a lookup
-// (two rows per wavefront instruction, padded onto different banks) never conflict.
+// workgroup stages the LUT rows of its row slice and K range in LDS, group-major, every 16-bit
+// value widened to a dword that holds it in both halves (rows 64 bytes apart), and a weight is one
+// 32-bit read at (code * 4) in its row; two reads are joined with one bit-field insert.  (16-bit
+// LDS reads of a half-size table measured four times slower per read than 32-bit ones.)  A row is
+// sixteen dwords on sixteen different banks and equal dwords are broadcast, so the lanes of a
+// lookup (two rows per wavefront instruction, padded onto the other sixteen banks) do not conflict.
 template <int LPGL, int NW, int PF, bool BF16, bool WALK = false, int BA = 4, int BB = 4, bool KG = false>
 __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -233,7 +235,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     constexpr bool TWO = !(BA == 4 && BB == 4);     // two resident tables
     static_assert(!TWO || !WALK, "walking grids: the (4, 4) kernel");
     static_assert(!KG || (!TWO && !WALK), "K-grouped LUTs: one 4-bit stream, one slice per workgroup");
-    constexpr int KG_GROUP = RW * 32 + (RW / 8) * 32;   // LDS bytes of one K group's rows
+    constexpr int KG_GROUP = RW * 64 + (RW / 8) * 64;   // LDS bytes of one K group's rows
     constexpr int TAB_A = (1 << (2 * BA)) * STRIDE; // bytes of the first table
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
@@ -396,8 +398,16 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 #pragma unroll
             for (int i = 0; i < KG_MAX; ++i) {
                 if (i * NT < kg_pieces) {
-                    if (r < RW)
-                        *(uint4 *)(lds + (pc >> 1) * KG_GROUP + r * 32 + (r >> 3) * 32 + (pc & 1) * 16) = slab_v[i];
+                    if (r < RW) {
+                        // eight 16-bit values -> eight dwords, each value in both halves
+                        const uint4 v = slab_v[i];
+                        auto both = [](uint32_t two, int hi) -> uint32_t {
+                            return hi ? (two >> 16) | (two & 0xffff0000u) : (two & 0xffffu) | (two << 16);
+                        };
+                        uint8_t *dst = lds + (pc >> 1) * KG_GROUP + r * 64 + (r >> 3) * 64 + (pc & 1) * 32;
+                        *(uint4 *)dst = make_uint4(both(v.x, 0), both(v.x, 1), both(v.y, 0), both(v.y, 1));
+                        *(uint4 *)(dst + 16) = make_uint4(both(v.z, 0), both(v.z, 1), both(v.w, 0), both(v.w, 1));
+                    }
                     r += kg_dr;
                     pc += kg_dp;
                     if (pc >= kg_row_pieces) {
@@ -664,22 +674,59 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // per row group v, eight lookups feed two matrix products; pair pp = v * 4 + d * 2 + s2 of a
     // quarter, an operand is (s2 = 0, 1) of both units
     // (K-grouped LUT: ga, gb = LDS byte offsets of the two units' K groups plus this lane's rows)
-    typedef const __attribute__((address_space(3))) uint16_t *LdsHalf;
     auto unit_pair = [&](const auto &qa, const auto &qb, gv_u4_t Bop, uint32_t tslot, auto width,
                          uint32_t ga = 0, uint32_t gb = 0) {
         constexpr int B = decltype(width)::value;
+        if constexpr (KG) {
+            // Row group v needs sixteen 16-bit reads (dword v of both units: four bytes of two
+            // codes).  Their addresses are formed while the reads of group v - 1 are in flight, and
+            // the reads go out behind that group's products: address arithmetic, LDS round trip
+            // and matrix products of neighbouring groups overlap instead of following each other.
+            auto addresses = [&](int v, uint32_t (&ad)[16]) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint32_t wq = u ? qb.d[v] : qa.d[v];
+                    const uint32_t base = (u ? gb : ga) + (uint32_t)(2 * v * 64);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        // byte j of the dword: row 2 v + (j >> 1), the two codes of one pair
+                        const uint32_t row = base + (uint32_t)((j >> 1) * 64);
+                        ad[u * 8 + j * 2] = (__builtin_amdgcn_ubfe(wq, 8 * j, 4) << 2) + row;
+                        ad[u * 8 + j * 2 + 1] = (__builtin_amdgcn_ubfe(wq, 8 * j + 4, 4) << 2) + row;
+                    }
+                }
+            };
+            auto reads = [&](const uint32_t (&ad)[16], uint32_t (&r)[16]) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) r[i] = *(LdsWord)ad[i];
+            };
+            auto products = [&](int v, const uint32_t (&r)[16]) {
+                // (every dword holds its value in both halves: low half of one, high half of the other)
+                auto pr = [&](int i) -> uint32_t { return (r[2 * i] & 0xffffu) | (r[2 * i + 1] & 0xffff0000u); };
+                // pairs 0..3: unit a, bytes 0..3; pairs 4..7: unit b
+                const gv_u4_t A0 = {pr(0), pr(1), pr(4), pr(5)};
+                const gv_u4_t A1 = {pr(2), pr(3), pr(6), pr(7)};
+                acc[v * 2] = gv_mfma<BF16>(A0, Bop, acc[v * 2]);
+                acc[v * 2 + 1] = gv_mfma<BF16>(A1, Bop, acc[v * 2 + 1]);
+            };
+            uint32_t ad[16], r[16];
+            addresses(0, ad);
+            reads(ad, r);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if (v < 3) addresses(v + 1, ad);
+                __builtin_amdgcn_sched_barrier(0);
+                products(v, r);
+                __builtin_amdgcn_sched_barrier(0);
+                if (v < 3) reads(ad, r);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            return;
+        }
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            auto look = [&](const IdxQuarter<B> &qq, int j, uint32_t goff = 0) -> uint32_t {
-                if constexpr (KG) {
-                    // byte j of dword v: rows a = 2 v + (j >> 1); the two codes of the pair are
-                    // two 16-bit reads in that row of the unit's K group
-                    const uint32_t base = goff + (uint32_t)((2 * v + (j >> 1)) * 32);
-                    const uint32_t c0 = __builtin_amdgcn_ubfe(qq.d[v], 8 * j, 4);
-                    const uint32_t c1 = __builtin_amdgcn_ubfe(qq.d[v], 8 * j + 4, 4);
-                    const uint32_t lo = *(LdsHalf)((c0 << 1) + base), hi = *(LdsHalf)((c1 << 1) + base);
-                    return lo | (hi << 16);
-                } else if constexpr (B == 4 && !TWO) {
+            auto look = [&](const IdxQuarter<B> &qq, int j) -> uint32_t {
+                if constexpr (B == 4 && !TWO) {
                     // a whole byte of dword v; byte 0: shift, then one and-or (the slot lies
                     // below the stride, the table at offset 0)
                     const uint32_t wq = qq.d[v];
@@ -689,8 +736,8 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                     return *(LdsWord)((quarter_code<B>(qq, v * 4 + j) << ES) + tslot);
                 }
             };
-            const gv_u4_t A0 = {look(qa, 0, ga), look(qa, 1, ga), look(qb, 0, gb), look(qb, 1, gb)};
-            const gv_u4_t A1 = {look(qa, 2, ga), look(qa, 3, ga), look(qb, 2, gb), look(qb, 3, gb)};
+            const gv_u4_t A0 = {look(qa, 0), look(qa, 1), look(qb, 0), look(qb, 1)};
+            const gv_u4_t A1 = {look(qa, 2), look(qa, 3), look(qb, 2), look(qb, 3)};
             acc[v * 2] = gv_mfma<BF16>(A0, Bop, acc[v * 2]);
             acc[v * 2 + 1] = gv_mfma<BF16>(A1, Bop, acc[v * 2 + 1]);
         }
@@ -699,7 +746,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // tiles per group) plus this lane's first row (chunk group cgl: eight rows and one pad).
     auto kg_off = [&](int m) -> uint32_t {
         if constexpr (!KG) return 0u;
-        return (uint32_t)((((w + m * NW) * GPI + gsub) >> 1) * KG_GROUP + cgl * (8 * 32 + 32));
+        return (uint32_t)((((w + m * NW) * GPI + gsub) >> 1) * KG_GROUP + cgl * (8 * 64 + 64));
     };
     // The K range of one stream of width B held in qc, refilled from qcur; the last group's
     // registers are refilled with the first loads of what follows: a stream of width BN from
