@@ -59,7 +59,10 @@ typedef enum flute_dtype {
  * LUT entry exactly.  bfloat16 activations with a float16 LUT are scaled by a power of
  * two per staged row (exact) on their way into the kernel and the row sums are scaled
  * back, so activations beyond float16's range (|x| > 65504, |x| < 6e-8) give the same
- * result as fp32 arithmetic on x.float().  float16 activations with a bfloat16 LUT are
+ * result as fp32 arithmetic on x.float().  A row that holds an infinity or a NaN is not
+ * scaled (there is no finite maximum to scale by): its finite values beyond float16's range
+ * saturate, so the outputs of such a row are unspecified (they may be NaN where fp32
+ * arithmetic gives an infinity).  float16 activations with a bfloat16 LUT are
  * refused (FLUTE_ERR_UNSUPPORTED): that conversion is not exact.
  * signs   (K,) fp32 +-1: when non-NULL the input is rotated first, x <- x @ T
  *         (fht.py:19-35); awq (K,) fp32 then selects ((x*s) @ T) / s
