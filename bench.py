@@ -301,7 +301,19 @@ def _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, down, keep_down,
         two.append(d)
         keep2.append((q2, l2))
     out["gemv_4096x12288_two_streams_4_1"] = gv.run("two_streams", two, keep, I, H, x, keep2=keep2, bits2=1)
-    del two, keep2
+    # (1, 4): the same operands with the streams in the other order (upstream's most frequent pair)
+    one_four = []
+    for d4, (q1b, l1b) in zip(gate, keep2):
+        d = _copy_desc(_lib, ctypes, d4)
+        d.q2, d.lut2, d.q2_bytes, d.b2 = d4.q1, d4.lut1, d4.q1_bytes, 4
+        d.q1, d.lut1, d.q1_bytes, d.b1 = q1b.data_ptr(), l1b.data_ptr(), q1b.numel(), 1
+        one_four.append(d)
+    both = lambda t: (_oracle_rows(O, keep[0][0], keep[0][1], H, t) +
+                      _oracle_rows(O, keep2[0][0], keep2[0][1], H, t, 1))
+    out["gemv_4096x12288_two_streams_1_4"] = gv.run(
+        "two_streams_1_4", one_four, keep, I, H, x, rows_of=both,
+        wbytes=I * H // 2 + (I // GS) * 32 + I * H // 8 + (I // GS) * 4)
+    del two, keep2, one_four
     # LUT grouped along K: one row of 16 values per (output row, 128-wide K group), [N, K/128, 16]
     # (a form no upstream artifact has; bytes = indices + that LUT = 37,748,736 at 4096 -> 12288)
     def k_grouped(name, descs, blobs, N, K, xin):
