@@ -213,7 +213,13 @@ constexpr int kKGroupPieces = 8;
 // LDS reads of a half-size table measured four times slower per read than 32-bit ones.)  A row is
 // sixteen dwords on sixteen different banks and equal dwords are broadcast, so the lanes of a
 // lookup (two rows per wavefront instruction, padded onto the other sixteen banks) do not conflict.
-template <int LPGL, int NW, int PF, bool BF16, bool WALK = false, int BA = 4, int BB = 4, bool KG = false>
+// DEEP (two tables, PF = 4, a 1-bit first stream): that stream keeps eight loads in flight instead
+// of four.  Its loads are four bytes per lane, so a group of four is consumed long before its
+// refill can be back; the deeper ring costs four registers.  The host picks it when a wavefront's
+// loads are a multiple of eight ((1, 4) at 4096 -> 12288: 10.5 -> 9.7 us; with the 1-bit stream
+// second it measured no gain, so the host puts it first).
+template <int LPGL, int NW, int PF, bool BF16, bool WALK = false, int BA = 4, int BB = 4, bool KG = false,
+          bool DEEP = false>
 __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     constexpr int ES = 7;
@@ -235,6 +241,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     constexpr bool TWO = !(BA == 4 && BB == 4);     // two resident tables
     static_assert(!TWO || !WALK, "walking grids: the (4, 4) kernel");
     static_assert(!KG || (!TWO && !WALK), "K-grouped LUTs: one 4-bit stream, one slice per workgroup");
+    static_assert(!DEEP || (TWO && PF == 4 && BA == 1), "the deep ring is for a 1-bit first stream");
+    constexpr int DA = (DEEP && BA == 1) ? 2 * PF : PF;  // loads in flight, first / second stream
+    constexpr int DB = (DEEP && BB == 1) ? 2 * PF : PF;
     constexpr int KG_GROUP = RW * 64 + (RW / 8) * 64;   // LDS bytes of one K group's rows
     constexpr int TAB_A = (1 << (2 * BA)) * STRIDE; // bytes of the first table
 
@@ -323,9 +332,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // plus one lane-constant 32-bit offset, so no per-load address lives in vector
     // registers; every load is unconditional, so the compiler knows how many are in
     // flight at each point and waits for exactly the ones a product needs.
-    auto first_units = [&](const uint8_t *qr, IdxQuarter<BA> (&qq)[PF], int from) {
+    auto first_units = [&](const uint8_t *qr, IdxQuarter<BA> (&qq)[DA], int from) {
 #pragma unroll
-        for (int n = 0; n < PF; ++n) {
+        for (int n = 0; n < DA; ++n) {
             if (n >= from) {
                 qq[n] = load_idx<BA>(qr + (size_t)n * step + lane0);
                 __builtin_amdgcn_sched_barrier(0);  // issue order = consumption order
@@ -481,8 +490,8 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     const uint16_t *staged_x = kp->seg[si0].xsrc ? kp->seg[si0].xsrc : p.x;
     const float *staged_signs = kp->seg[si0].signs, *staged_awq = kp->seg[si0].awq;
     const bool x_plain = staged_signs == nullptr;   // plain copy
-    IdxQuarter<BA> q[PF];
-    IdxQuarter<BB> q2[PF];
+    IdxQuarter<BA> q[DA];
+    IdxQuarter<BB> q2[DB];
     // bfloat16 activations in front of a float16 LUT: the staged units hold x * 2^-xshift,
     // xshift chosen per wavefront (per workgroup when the input is rotated)
     const bool convert = !BF16 && p.act_bf16;       // uniform
@@ -753,40 +762,46 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // qnext into qn (nothing when last).
     auto k_loop = [&](auto &qc, const uint8_t *qcur, uint32_t lane_c, uint32_t step_c, uint32_t tslot,
                       auto width, auto &qn, const uint8_t *qnext, uint32_t lane_n, uint32_t step_n,
-                      auto width_next, bool has_next) {
+                      auto width_next, bool has_next, bool output_ends = true) {
         constexpr int B = decltype(width)::value, BN = decltype(width_next)::value;
+        // the ring depths are the extents of the register arrays
+        constexpr int D = (int)(sizeof(qc) / sizeof(qc[0])), DN = (int)(sizeof(qn) / sizeof(qn[0]));
         int nb = 0;
         __builtin_amdgcn_s_setprio(2);
-        for (; nb + 2 * PF <= my_units; nb += PF) {          // every refill exists
+        for (; nb + 2 * D <= my_units; nb += D) {            // every refill exists
 #pragma unroll
-            for (int n = 0; n < PF; n += 2) {
+            for (int n = 0; n < D; n += 2) {
                 const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
                 unit_pair(qc[n], qc[n + 1], Bop, tslot, width, kg_off(nb + n), kg_off(nb + n + 1));
                 __builtin_amdgcn_sched_barrier(0);
-                qc[n] = load_idx<B>(qcur + (size_t)(nb + n + PF) * step_c + lane_c);
-                qc[n + 1] = load_idx<B>(qcur + (size_t)(nb + n + 1 + PF) * step_c + lane_c);
+                qc[n] = load_idx<B>(qcur + (size_t)(nb + n + D) * step_c + lane_c);
+                qc[n + 1] = load_idx<B>(qcur + (size_t)(nb + n + 1 + D) * step_c + lane_c);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (!has_next) __builtin_amdgcn_s_setprio(1);
+        if (!has_next && output_ends) __builtin_amdgcn_s_setprio(1);
         if (has_next) {
 #pragma unroll
-            for (int n = 0; n < PF; n += 2) {
+            for (int n = 0; n < D; n += 2) {
                 const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
                 unit_pair(qc[n], qc[n + 1], Bop, tslot, width, kg_off(nb + n), kg_off(nb + n + 1));
                 __builtin_amdgcn_sched_barrier(0);
-                qn[n] = load_idx<BN>(qnext + (size_t)n * step_n + lane_n);
-                qn[n + 1] = load_idx<BN>(qnext + (size_t)(n + 1) * step_n + lane_n);
+                if (n < DN) {
+                    qn[n] = load_idx<BN>(qnext + (size_t)n * step_n + lane_n);
+                    qn[n + 1] = load_idx<BN>(qnext + (size_t)(n + 1) * step_n + lane_n);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
+#pragma unroll
+            for (int n = D; n < DN; ++n) qn[n] = load_idx<BN>(qnext + (size_t)n * step_n + lane_n);
         } else {
 #pragma unroll
-            for (int n = 0; n < PF; n += 2) {
+            for (int n = 0; n < D; n += 2) {
                 const gv_u4_t Bop = operand_b(nb + n, nb + n + 1);
                 unit_pair(qc[n], qc[n + 1], Bop, tslot, width, kg_off(nb + n), kg_off(nb + n + 1));
             }
         }
-        if (!has_next) __builtin_amdgcn_s_setprio(0);
+        if (!has_next && output_ends) __builtin_amdgcn_s_setprio(0);
     };
     // ---- end of an output: D[i][j] with i = (rb, kt) in (lane >> 4, register) and
     //      j = (rb', kt') in lane & 15.  The lanes with rb' == rb keep register kt';
@@ -829,9 +844,18 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                     load_lut_row<BB>(lutn, lrowB);
                 }
             }
+            // the second stream's first loads go out before the first stream's loop: its registers
+            // are free from here on, and its data is then there when its loop starts
+            if (second) {
+#pragma unroll
+                for (int n = 0; n < DB; ++n) {
+                    q2[n] = load_idx<BB>(qb_cur + (size_t)n * stepB + lane0B);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
             __syncthreads();                        // publishes the tables (and the staged activations)
             if (second) {
-                k_loop(q, qrow, lane0, step, slot, WA, q2, qb_cur, lane0B, stepB, WB, true);
+                k_loop(q, qrow, lane0, step, slot, WA, q2, qb_cur, lane0B, stepB, WB, false, false);
                 k_loop(q2, qb_cur, lane0B, stepB, slotB, WB, q, qa_next, lane0, step, WA, more);
             } else {
                 k_loop(q, qrow, lane0, step, slot, WA, q, qa_next, lane0, step, WA, more);
