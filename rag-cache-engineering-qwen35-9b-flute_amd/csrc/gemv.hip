@@ -357,7 +357,9 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
         const int code = 10 * b1 + b2;
         if (ok && (code == 41 || code == 14 || code == 33)) {
             plan->pair = code;
-            const size_t both = (((size_t)1 << (2 * b1)) + ((size_t)1 << (2 * b2))) * 128;
+            // (4^b entries of 128 bytes; a 1-bit stream's nibble table: 16 entries of 256 bytes)
+            auto tab = [](int b) { return b == 1 ? (size_t)16 * 256 : ((size_t)1 << (2 * b)) * 128; };
+            const size_t both = tab(b1) + tab(b2);
             if (both > tab_bytes) tab_bytes = both;
             // (4, 1) where every weight has both streams: the kernel walks the 1-bit stream first
             // (the sum of the two streams does not depend on their order beyond fp32 rounding, and

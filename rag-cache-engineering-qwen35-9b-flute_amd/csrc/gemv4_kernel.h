@@ -245,7 +245,11 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     constexpr int DA = (DEEP && BA == 1) ? 2 * PF : PF;  // loads in flight, first / second stream
     constexpr int DB = (DEEP && BB == 1) ? 2 * PF : PF;
     constexpr int KG_GROUP = RW * 64 + (RW / 8) * 64;   // LDS bytes of one K group's rows
-    constexpr int TAB_A = (1 << (2 * BA)) * STRIDE; // bytes of the first table
+    // A 1-bit stream (two tables only) is looked up a nibble at a time: four weights of one row =
+    // two operand dwords from one 8-byte entry, sixteen entries, 32 replicas 8 bytes apart (4 KB).
+    // Half the lookups and address instructions of the pair-at-a-time form.
+    constexpr int TAB1 = 16 * 256;
+    constexpr int TAB_A = (TWO && BA == 1) ? TAB1 : (1 << (2 * BA)) * STRIDE;  // bytes of the first table
 
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     warm_kernargs<(int)sizeof(GemvParams)>(kp);
@@ -309,7 +313,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // address of byte 0 be formed as shift + and-or, two instructions like the other bytes.
     __builtin_assume(lds_base == 0);
     const uint32_t slot = lds_base + (uint32_t)(L & 31) * 4u;
-    const uint32_t slotB = slot + (TWO ? TAB_A : 0);
+    const uint32_t slot1 = lds_base + (uint32_t)(L & 31) * 8u;       // (nibble table of a 1-bit stream)
+    const uint32_t slotA = (TWO && BA == 1) ? slot1 : slot;
+    const uint32_t slotB = ((TWO && BB == 1) ? slot1 : slot) + (TWO ? TAB_A : 0);
     const int e_own = tid & 255;                    // table entry this thread writes
     const int share = tid >> 8;
 
@@ -356,6 +362,17 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // the replicas of its entry.
     auto write_small_table = [&](const uint32_t (&row)[8], auto width, uint32_t base) {
         constexpr int B = decltype(width)::value;
+        if constexpr (B == 1) {
+            if (tid < 16) {                         // entry = four bits b0..b3 -> {l[b0] l[b1]} {l[b2] l[b3]}
+                const uint32_t lo = lut_value(row, tid & 1) | (lut_value(row, (tid >> 1) & 1) << 16);
+                const uint32_t hi = lut_value(row, (tid >> 2) & 1) | (lut_value(row, tid >> 3) << 16);
+                const uint4 v4 = make_uint4(lo, hi, lo, hi);
+                uint8_t *ent = lds + base + tid * 256;
+#pragma unroll
+                for (int k = 0; k < 16; ++k) *(uint4 *)(ent + (((k + tid) & 15) << 4)) = v4;
+            }
+            return;
+        }
         if (tid < (1 << (2 * B))) {
             const uint32_t v = lut_value(row, tid & ((1 << B) - 1)) | (lut_value(row, tid >> B) << 16);
             const uint4 v4 = make_uint4(v, v, v, v);
@@ -732,6 +749,24 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             }
             return;
         }
+        if constexpr (B == 1) {
+            typedef uint32_t pair_t __attribute__((ext_vector_type(2)));
+            typedef const __attribute__((address_space(3))) pair_t *LdsPair;
+            const uint32_t wa = qa.d[0], wb = qb.d[0];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                // byte v of the quarter: low nibble = the four weights of row 2 v, high nibble = row 2 v + 1
+                const pair_t a0 = *(LdsPair)((__builtin_amdgcn_ubfe(wa, 8 * v, 4) << 8) + tslot);
+                const pair_t a1 = *(LdsPair)((__builtin_amdgcn_ubfe(wa, 8 * v + 4, 4) << 8) + tslot);
+                const pair_t b0 = *(LdsPair)((__builtin_amdgcn_ubfe(wb, 8 * v, 4) << 8) + tslot);
+                const pair_t b1 = *(LdsPair)((__builtin_amdgcn_ubfe(wb, 8 * v + 4, 4) << 8) + tslot);
+                const gv_u4_t A0 = {a0.x, a0.y, b0.x, b0.y};
+                const gv_u4_t A1 = {a1.x, a1.y, b1.x, b1.y};
+                acc[v * 2] = gv_mfma<BF16>(A0, Bop, acc[v * 2]);
+                acc[v * 2 + 1] = gv_mfma<BF16>(A1, Bop, acc[v * 2 + 1]);
+            }
+            return;
+        }
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             auto look = [&](const IdxQuarter<B> &qq, int j) -> uint32_t {
@@ -855,10 +890,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             }
             __syncthreads();                        // publishes the tables (and the staged activations)
             if (second) {
-                k_loop(q, qrow, lane0, step, slot, WA, q2, qb_cur, lane0B, stepB, WB, false, false);
+                k_loop(q, qrow, lane0, step, slotA, WA, q2, qb_cur, lane0B, stepB, WB, false, false);
                 k_loop(q2, qb_cur, lane0B, stepB, slotB, WB, q, qa_next, lane0, step, WA, more);
             } else {
-                k_loop(q, qrow, lane0, step, slot, WA, q, qa_next, lane0, step, WA, more);
+                k_loop(q, qrow, lane0, step, slotA, WA, q, qa_next, lane0, step, WA, more);
             }
             end_of_output(so, 0);
             if (!more) break;
