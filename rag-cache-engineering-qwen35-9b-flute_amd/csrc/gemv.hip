@@ -355,7 +355,7 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
             }
         }
         const int code = 10 * b1 + b2;
-        if (ok && (code == 41 || code == 14 || code == 33)) {
+        if (ok && (code == 41 || code == 14 || code == 33 || code == 24 || code == 23)) {
             plan->pair = code;
             // (4^b entries of 128 bytes; a 1-bit stream's nibble table: 16 entries of 256 bytes)
             auto tab = [](int b) { return b == 1 ? (size_t)16 * 256 : ((size_t)1 << (2 * b)) * 128; };
@@ -576,6 +576,8 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         switch (plan.pair) {
             case 41: return launch_pair<BF16, 4, 1>(plan, nw, pf, stream);
             case 14: return launch_pair<BF16, 1, 4>(plan, nw, pf, stream);
+            case 24: return launch_pair<BF16, 2, 4>(plan, nw, pf, stream);
+            case 23: return launch_pair<BF16, 2, 3>(plan, nw, pf, stream);
             default: return launch_pair<BF16, 3, 3>(plan, nw, pf, stream);
         }
     }

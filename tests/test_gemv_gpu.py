@@ -510,7 +510,7 @@ PAIR_SHAPES = [
 
 
 @pytest.mark.parametrize("act", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3)])
+@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3), (2, 4), (2, 3)])
 @pytest.mark.parametrize("N,K", PAIR_SHAPES)
 def test_width_pairs_two_resident_tables(N, K, bits, bits2, act):
     """Every row against the fp64 oracle at the reference forward's rounding point, repeats bit
@@ -525,7 +525,7 @@ def test_width_pairs_two_resident_tables(N, K, bits, bits2, act):
     assert torch.equal(y, _run(w, x).cpu())
 
 
-@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3)])
+@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3), (2, 4), (2, 3)])
 def test_width_pairs_one_hot_rows_are_the_sum_of_both_dequantised_columns(bits, bits2):
     """x = e_k: the output is W1[:, k] + W2[:, k], one fp32 add of two 16-bit values rounded once:
     bit-exact against the dequantised columns for k in every quarter of a tile."""
@@ -541,7 +541,7 @@ def test_width_pairs_one_hot_rows_are_the_sum_of_both_dequantised_columns(bits, 
 
 
 @pytest.mark.parametrize("split", [2, 4])
-@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3)])
+@pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3), (2, 4), (2, 3)])
 def test_width_pairs_with_a_k_split_residual_and_bias(bits, bits2, split):
     w = make_weight(1024, 4096, bits, 128, seed=9, bits2=bits2, rank=8, bias=True, device=DEV)
     x = make_x(1, 4096, seed=4)
