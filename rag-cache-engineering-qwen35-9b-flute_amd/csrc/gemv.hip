@@ -354,7 +354,13 @@ flute_status make_plan(const flute_linear *segs, int count, const void *x, void 
                 ok &= segs[i].b2 == b2;
             }
         }
-        const int code = 10 * b1 + b2;
+        int code = 10 * b1 + b2;
+        // a single narrow stream ((3, 0) is one of upstream's pairs): the two-table instantiation
+        // of its width with the second table unused
+        if (b2 == 0 && b1 < 4) {
+            b2 = b1 == 3 ? 3 : (b1 == 2 ? 3 : 4);
+            code = 10 * b1 + b2;
+        }
         if (ok && (code == 41 || code == 14 || code == 33 || code == 24 || code == 23)) {
             plan->pair = code;
             // (4^b entries of 128 bytes; a 1-bit stream's nibble table: 16 entries of 256 bytes)
