@@ -452,55 +452,6 @@ flute_status launch_fast4(Plan &plan, hipStream_t stream) {
     return launch_fast4_grid<LPGL, NW, PF, BF16, false>(plan, gx, stream);
 }
 
-// The lean kernel with two resident tables (mixed widths); no walking grid.  Eight wavefronts
-// come with 8- or 16-row slices only (choose_shape).
-template <int LPGL, int NW, int PF, bool BF16, int BA, int BB, bool DEEP = false>
-flute_status launch_pair_grid(const Plan &plan, hipStream_t stream) {
-    static std::atomic<bool> attr_done{false};
-    if (!attr_done) {
-        FLUTE_HIP_CHECK(hipFuncSetAttribute(
-            (const void *)gemv4_kernel<LPGL, NW, PF, BF16, false, BA, BB, false, DEEP>,
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerCU));
-        attr_done = true;
-    }
-    dim3 grid(plan.grid_x, plan.p.split);
-    hipLaunchKernelGGL((gemv4_kernel<LPGL, NW, PF, BF16, false, BA, BB, false, DEEP>), grid, dim3(NW * 64),
-                       plan.lds_bytes, stream, plan.p);
-    FLUTE_HIP_CHECK(hipGetLastError());
-    return FLUTE_OK;
-}
-// pf: 2 or 4; 8 = four with the deep ring for the 1-bit stream of the pair (a wavefront's loads
-// are then a multiple of eight)
-template <bool BF16, int BA, int BB>
-flute_status launch_pair(Plan &plan, int nw, int pf, hipStream_t stream) {
-    plan.p.slices = 0;
-    constexpr bool NARROW = BA == 1;                 // the deep ring: for a 1-bit stream in front
-    switch (nw * 100 + plan.p.lpg_log2 * 10 + pf) {
-        case 442: return launch_pair_grid<4, 4, 2, BF16, BA, BB>(plan, stream);
-        case 444: return launch_pair_grid<4, 4, 4, BF16, BA, BB>(plan, stream);
-        case 452: return launch_pair_grid<5, 4, 2, BF16, BA, BB>(plan, stream);
-        case 454: return launch_pair_grid<5, 4, 4, BF16, BA, BB>(plan, stream);
-        case 462: return launch_pair_grid<6, 4, 2, BF16, BA, BB>(plan, stream);
-        case 464: return launch_pair_grid<6, 4, 4, BF16, BA, BB>(plan, stream);
-        case 842: return launch_pair_grid<4, 8, 2, BF16, BA, BB>(plan, stream);
-        case 844: return launch_pair_grid<4, 8, 4, BF16, BA, BB>(plan, stream);
-        case 852: return launch_pair_grid<5, 8, 2, BF16, BA, BB>(plan, stream);
-        case 854: return launch_pair_grid<5, 8, 4, BF16, BA, BB>(plan, stream);
-        default: break;
-    }
-    if constexpr (NARROW) {
-        switch (nw * 100 + plan.p.lpg_log2 * 10 + pf) {
-            case 448: return launch_pair_grid<4, 4, 4, BF16, BA, BB, true>(plan, stream);
-            case 458: return launch_pair_grid<5, 4, 4, BF16, BA, BB, true>(plan, stream);
-            case 468: return launch_pair_grid<6, 4, 4, BF16, BA, BB, true>(plan, stream);
-            case 848: return launch_pair_grid<4, 8, 4, BF16, BA, BB, true>(plan, stream);
-            case 858: return launch_pair_grid<5, 8, 4, BF16, BA, BB, true>(plan, stream);
-            default: break;
-        }
-    }
-    return FLUTE_ERR_UNSUPPORTED;                    // (not reached: the caller checks the shape)
-}
-
 // Loads a lane keeps in flight in the lean kernel: 4 when that divides the loads of a
 // wavefront, else 2; 0 when the launch does not fit the kernel (the wavefronts would get
 // different or odd numbers of loads: two loads feed one matrix product).
@@ -579,13 +530,10 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         // a 1-bit stream with loads that come in eights: the deep ring (launch_pair's pf 8)
         const int u = (plan.p.gs_tiles / (64 >> plan.p.lpg_log2)) / nw;
         if (pf == 4 && plan.pair == 14 && u % 8 == 0 && tuning().gemv4_pf == 0) pf = 8;
-        switch (plan.pair) {
-            case 41: return launch_pair<BF16, 4, 1>(plan, nw, pf, stream);
-            case 14: return launch_pair<BF16, 1, 4>(plan, nw, pf, stream);
-            case 24: return launch_pair<BF16, 2, 4>(plan, nw, pf, stream);
-            case 23: return launch_pair<BF16, 2, 3>(plan, nw, pf, stream);
-            default: return launch_pair<BF16, 3, 3>(plan, nw, pf, stream);
-        }
+        plan.p.slices = 0;
+        return (plan.pair == 41 || plan.pair == 14)
+                   ? launch_gemv_pair_1bit(plan.p, plan.pair, plan.grid_x, nw, pf, plan.lds_bytes, BF16, stream)
+                   : launch_gemv_pair_wide(plan.p, plan.pair, plan.grid_x, nw, pf, plan.lds_bytes, BF16, stream);
     }
     switch (bits) {
         case 4: return launch_typed<BF16, 4>(plan, stream);

@@ -1020,4 +1020,11 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
 flute_status launch_gemv_kgroup(const GemvParams &p, int grid_x, int nw, int pf, size_t lds_bytes,
                                 bool lut_bf16, hipStream_t stream);
 
+// The launches of the two-table instantiations (their own translation units).  pair = 10 * BA + BB;
+// pf: 2 or 4, 8 = four with the deep ring of a 1-bit first stream.
+flute_status launch_gemv_pair_1bit(const GemvParams &p, int pair, int grid_x, int nw, int pf,
+                                   size_t lds_bytes, bool lut_bf16, hipStream_t stream);
+flute_status launch_gemv_pair_wide(const GemvParams &p, int pair, int grid_x, int nw, int pf,
+                                   size_t lds_bytes, bool lut_bf16, hipStream_t stream);
+
 }  // namespace flute
