@@ -540,6 +540,19 @@ def test_width_pairs_one_hot_rows_are_the_sum_of_both_dequantised_columns(bits, 
         assert torch.equal(y[0], (W1[:, k].float() + W2[:, k].float()).half())
 
 
+def test_a_4_1_weight_equals_the_same_weight_declared_1_4():
+    """The library walks a 1-bit stream first whichever way the weight declares its streams: the
+    two declarations of the same data must agree bit for bit (and both with the oracle)."""
+    N, K = 12288, 4096
+    w = make_weight(N, K, 4, 128, seed=77, bits2=1, device=DEV)
+    x = make_x(1, K, seed=19)
+    y41 = _run(w, x)
+    y14 = fx.qgemm_gemv_splitk_stream(x.to(DEV), w["blob2_d"], w["lut2_d"], 1, 128, indices2=w["blob_d"],
+                                      lut2=w["lut_d"], bitwidth2=4)
+    assert torch.equal(y41, y14)
+    assert rel_l2(y41.cpu(), _exact(w, x).half()) <= TOL
+
+
 @pytest.mark.parametrize("split", [2, 4])
 @pytest.mark.parametrize("bits,bits2", [(4, 1), (1, 4), (3, 3), (2, 4), (2, 3)])
 def test_width_pairs_with_a_k_split_residual_and_bias(bits, bits2, split):
