@@ -313,7 +313,7 @@ def _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, down, keep_down,
     out["gemv_4096x12288_two_streams_1_4"] = gv.run(
         "two_streams_1_4", one_four, keep, I, H, x, rows_of=both,
         wbytes=I * H // 2 + (I // GS) * 32 + I * H // 8 + (I // GS) * 4)
-    del two, keep2, one_four
+    del two
     # LUT grouped along K: one row of 16 values per (output row, 128-wide K group), [N, K/128, 16]
     # (a form no upstream artifact has; bytes = indices + that LUT = 37,748,736 at 4096 -> 12288)
     def k_grouped(name, descs, blobs, N, K, xin):
@@ -358,6 +358,12 @@ def _other_m1(torch, _lib, ctypes, O, dev, gen, gv, gate, keep, down, keep_down,
         xref=O.block_fht_reference(x.cpu(), 128, signs.cpu()).to(x.dtype))
     out["gemv_4096x12288_fht_full_k_fused"] = gv.run(
         "fht_full_k_up", rotated(gate, signs, 0), keep, I, H, x, xref=O.fht_reference(x.cpu(), signs.cpu()))
+    # what a deployed weight is: a (1, 4) pair behind upstream's full-K rotation
+    out["gemv_4096x12288_two_streams_1_4_fht_full_k_fused"] = gv.run(
+        "two_streams_1_4_fht_full_k", rotated(one_four, signs, 0), keep, I, H, x,
+        xref=O.fht_reference(x.cpu(), signs.cpu()), rows_of=both,
+        wbytes=I * H // 2 + (I // GS) * 32 + I * H // 8 + (I // GS) * 4)
+    del keep2, one_four
     out["gemv_12288x4096_plain"] = gv.run("down_plain", down, keep_down, H, I, xd_)
     out["gemv_12288x4096_fht_full_k_fused"] = gv.run(
         "fht_full_k_down", rotated(down, signs_d, 0), keep_down, H, I, xd_,
