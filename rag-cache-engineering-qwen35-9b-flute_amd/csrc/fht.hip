@@ -106,13 +106,13 @@ __device__ __forceinline__ void store_cols8(const FhtParams &p, int64_t orow, in
     uint16_t op[8];
     float t[8];
 #pragma unroll
+    for (int q = 0; q < 8; ++q) t[q] = p.adjoint ? f[q] * inv : f[q] * sg[q] * inv;
+    if (!p.adjoint && p.awq) {          // one uniform branch: as a select per value every launch paid for the divisions
+#pragma unroll
+        for (int q = 0; q < 8; ++q) t[q] = t[q] / sc[q];
+    }
+#pragma unroll
     for (int q = 0; q < 8; ++q) {
-        if (p.adjoint) {
-            t[q] = f[q] * inv;
-        } else {
-            t[q] = f[q] * sg[q] * inv;
-            if (p.awq) t[q] = t[q] / sc[q];
-        }
         if (p.dtype != FLUTE_F32) {
             uint16_t a = round_act(t[q], bf16);
             if (p.ap && bf16 != p.ap_bf16) a = round_act(bf16 ? bf2f(a) : h2f(a), p.ap_bf16);
@@ -352,15 +352,19 @@ __global__ void __launch_bounds__(kFhtThreads) fht_kernel(const FhtParams p) {
         fht_lds(buf, count, nstages, tid, kFhtThreads);
         auto emit = [&](int j, const float (&sg)[8], const float (&sc)[8]) {
             uint16_t op[8];
+            float tt[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q) {
-                float t = buf[fht_slot(j + q)];
-                if (p.adjoint) {
-                    t = t * inv;
-                } else {
-                    t = t * sg[q] * inv;
-                    if (p.awq) t = t / sc[q];
-                }
+                const float b = buf[fht_slot(j + q)];
+                tt[q] = p.adjoint ? b * inv : b * sg[q] * inv;
+            }
+            if (!p.adjoint && p.awq) {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) tt[q] = tt[q] / sc[q];
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const float t = tt[q];
                 if (p.ap) {
                     const int in_bf16 = p.dtype == FLUTE_BF16;
                     uint16_t a = round_act(t, in_bf16);

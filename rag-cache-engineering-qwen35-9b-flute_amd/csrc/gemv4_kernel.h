@@ -176,14 +176,10 @@ __device__ __forceinline__ void rotate_piece(uint4 &v, const float (&sg)[8], con
     FLUTE_XOR_STAGE(16)
 #undef FLUTE_XOR_STAGE
     uint32_t o[4];
+    float t[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        float t = f[e] * sg[e] * inv;
-        if (has_awq) t = t / sc[e];
-        const uint32_t a = ACT_BF16 ? f2bf(t) : f2h(t);   // the standalone kernel's rounding
-        if (e & 1) o[e >> 1] |= a << 16;
-        else o[e >> 1] = a;
-    }
+    for (int e = 0; e < 8; ++e) t[e] = f[e] * sg[e] * inv;
+    pack_act8(t, has_awq ? sc : nullptr, ACT_BF16 ? 1 : 0, o);   // the standalone kernel's rounding
     v = make_uint4(o[0], o[1], o[2], o[3]);
 }
 

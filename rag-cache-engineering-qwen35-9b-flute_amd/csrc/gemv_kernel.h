@@ -291,6 +291,24 @@ __device__ __forceinline__ int normalise_staged_row(uint16_t *xs, int kc, uint32
     return shift;
 }
 
+// Eight rotated values, divided by the AWQ scales where there are any, rounded to the activation
+// type and packed.  The two conditions are uniform and sit outside the loops over the values: as
+// selects inside them (which is what an `if` around one division becomes) every launch paid for the
+// divisions and for both conversions, 25 vector instructions per value where 3 are needed.
+__device__ __forceinline__ void pack_act8(float (&t)[8], const float *sc, int act_bf16, uint32_t (&o)[4]) {
+    if (sc != nullptr) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) t[q] = t[q] / sc[q];
+    }
+    if (act_bf16) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) o[q] = (uint32_t)f2bf(t[2 * q]) | ((uint32_t)f2bf(t[2 * q + 1]) << 16);
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) o[q] = (uint32_t)f2h(t[2 * q]) | ((uint32_t)f2h(t[2 * q + 1]) << 16);
+    }
+}
+
 // Output side of the fused rotation, eight columns per step: value * sign * inv
 // (/ awq), rounded to the activation type exactly as the standalone kernel rounds,
 // then converted to the compute type.  The eight sign (and scale) loads of a step are
@@ -304,15 +322,10 @@ __device__ __forceinline__ void rotated_out8(const float *buf, int j, const floa
     if (awq) load_f8(awq, g, sc);
     uint32_t o[4];
     const int s0 = fht_slot(j);                        // j is a multiple of 8: slot(j + q) = s0 ^ q
+    float t[8];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-        float t = buf[s0 ^ q] * sg[q] * inv;
-        if (awq) t = t / sc[q];
-        const uint16_t a = round_act(t, act_bf16);
-        const uint32_t h = a;       // the activation type; the caller converts bf16 -> f16 if needed
-        if (q & 1) o[q >> 1] |= h << 16;
-        else o[q >> 1] = h;
-    }
+    for (int q = 0; q < 8; ++q) t[q] = buf[s0 ^ q] * sg[q] * inv;
+    pack_act8(t, awq ? sc : nullptr, act_bf16, o);
     *(uint4 *)dst = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
@@ -403,15 +416,10 @@ __device__ __forceinline__ void rotate_blocks_inwave(const uint16_t *x, const fl
         for (int h = 0; h < 2; ++h) {
             if (h == 1 && !two) break;
             uint32_t o[4];
+            float t[8];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                float t = f[h][q] * sg[h][q] * inv;
-                if (awq) t = t / sc[h][q];
-                const uint16_t a = round_act(t, act_bf16);
-                const uint32_t v = a;   // the activation type; the caller converts bf16 -> f16 if needed
-                if (q & 1) o[q >> 1] |= v << 16;
-                else o[q >> 1] = v;
-            }
+            for (int q = 0; q < 8; ++q) t[q] = f[h][q] * sg[h][q] * inv;
+            pack_act8(t, awq ? sc[h] : nullptr, act_bf16, o);   // (the activation type; the caller converts bf16 -> f16 if needed)
             *(uint4 *)(xs + (h ? j1 : j0)) = make_uint4(o[0], o[1], o[2], o[3]);
         }
     }
@@ -525,15 +533,10 @@ __device__ __forceinline__ void rotate_segment_fast(const uint16_t *x, const flo
         for (int h = 0; h < 2; ++h) {
             if (h == 1 && !two) break;
             uint32_t o[4];
+            float t[8];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                float t = f[h][q] * sg[h][q] * inv;
-                if (awq) t = t / sc[h][q];
-                const uint16_t a = round_act(t, act_bf16);
-                const uint32_t v = a;   // the activation type; the caller converts bf16 -> f16 if needed
-                if (q & 1) o[q >> 1] |= v << 16;
-                else o[q >> 1] = v;
-            }
+            for (int q = 0; q < 8; ++q) t[q] = f[h][q] * sg[h][q] * inv;
+            pack_act8(t, awq ? sc[h] : nullptr, act_bf16, o);   // (the activation type; the caller converts bf16 -> f16 if needed)
             *(uint4 *)(xs + xs_off + (h ? j1 : j0)) = make_uint4(o[0], o[1], o[2], o[3]);
         }
     }
