@@ -183,6 +183,21 @@ __device__ __forceinline__ void rotate_piece(uint4 &v, const float (&sg)[8], con
     v = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// a | byte J of w, in one instruction (the compiler's own choice is a shift and an and-or).
+template <int J>
+__device__ __forceinline__ uint32_t or_byte(uint32_t a, uint32_t w) {
+    uint32_t r;
+    if constexpr (J == 0)
+        asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(a), "v"(w));
+    else if constexpr (J == 1)
+        asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(a), "v"(w));
+    else if constexpr (J == 2)
+        asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(a), "v"(w));
+    else
+        asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(a), "v"(w));
+    return r;
+}
+
 // A LUT grouped along K: 16-byte pieces of LUT rows a thread stages at most.
 constexpr int kKGroupPieces = 8;
 
@@ -709,13 +724,19 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
                 for (int u = 0; u < 2; ++u) {
                     const uint32_t wq = u ? qb.d[v] : qa.d[v];
                     const uint32_t base = (u ? gb : ga) + (uint32_t)(2 * v * 64);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        // byte j of the dword: row 2 v + (j >> 1), the two codes of one pair
-                        const uint32_t row = base + (uint32_t)((j >> 1) * 64);
-                        ad[u * 8 + j * 2] = (__builtin_amdgcn_ubfe(wq, 8 * j, 4) << 2) + row;
-                        ad[u * 8 + j * 2 + 1] = (__builtin_amdgcn_ubfe(wq, 8 * j + 4, 4) << 2) + row;
-                    }
+                    // Entry offsets (code * 4) of the four low and the four high codes, one to a
+                    // byte: two instructions per set, then one byte-select OR per address (a row
+                    // of entries is 64 bytes and 64-byte aligned, so OR is the sum).
+                    const uint32_t lo = (wq << 2) & 0x3c3c3c3cu, hi = (wq >> 2) & 0x3c3c3c3cu;
+                    // byte j of the dword: row 2 v + (j >> 1), the two codes of one pair
+                    ad[u * 8 + 0] = or_byte<0>(base, lo);
+                    ad[u * 8 + 1] = or_byte<0>(base, hi);
+                    ad[u * 8 + 2] = or_byte<1>(base, lo);
+                    ad[u * 8 + 3] = or_byte<1>(base, hi);
+                    ad[u * 8 + 4] = or_byte<2>(base, lo) + 64u;
+                    ad[u * 8 + 5] = or_byte<2>(base, hi) + 64u;
+                    ad[u * 8 + 6] = or_byte<3>(base, lo) + 64u;
+                    ad[u * 8 + 7] = or_byte<3>(base, hi) + 64u;
                 }
             };
             auto reads = [&](const uint32_t (&ad)[16], uint32_t (&r)[16]) {
