@@ -495,6 +495,7 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         }
     }
     const int nw = plan.threads / 64;
+    plan.p.xcd_runs = tuning().gemv_xcd && (plan.p.nsegs == 1 || plan.p.silu_mul) && plan.grid_x % 8 == 0;
     // the lean kernel stages the activations once: gate and up must share input and rotation
     const bool one_input = !plan.p.silu_mul ||
                            (plan.p.seg[0].xsrc == plan.p.seg[1].xsrc &&

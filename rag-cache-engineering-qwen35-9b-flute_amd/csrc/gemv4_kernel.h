@@ -286,6 +286,13 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     // four slices of a tile at the same time, which the memory system likes better.
     constexpr bool walk = WALK;                     // unsplit launches of one column space
     int sl = (int)blockIdx.x - kp->seg[si0].col0;
+    if (!walk && p.xcd_runs) {
+        // Consecutive workgroups go to consecutive XCDs.  Every XCD takes a contiguous run of slices
+        // instead of every eighth one: the slices of a 128-row tile (their pieces of each 4 KB
+        // index tile, their LUT row) then meet in one L2.  Measured 1 - 5 % (most on narrow outputs).
+        const int b = (int)blockIdx.x, per = (int)gridDim.x >> 3;
+        sl = (b & 7) * per + (b >> 3);
+    }
     int sl_end = sl + 1, sl_step = 1;
     if constexpr (walk) {
         const int per = p.slices / (int)gridDim.x, extra = p.slices % (int)gridDim.x;

@@ -87,6 +87,7 @@ struct GemvParams {
     int lds_x;              // LDS byte offsets
     int lds_red;            // row sums [2][8][32] fp32, ticket flag (16 B), 8 words for a row maximum
     int slices;             // > 0: a workgroup walks the row slices blockIdx.x, + gridDim.x, ... below this
+    int xcd_runs;           // lean kernel, one column space: workgroup b takes slice (b % 8) * (grid / 8) + b / 8
 };
 
 // ---- small device helpers ---------------------------------------------------

@@ -241,6 +241,7 @@ static void read_tuning() {
     t.gemv4_pf = env_or("FLUTE_GEMV4_PF", 0);
     t.gemv_no_fast = env_or("FLUTE_GEMV_NO_FAST", 0);
     t.gemv4_walk = env_or("FLUTE_GEMV4_WALK", -1);
+    t.gemv_xcd = env_or("FLUTE_GEMV_XCD", 1);
     t.gemm_rows = env_or("FLUTE_GEMM_ROWS", 0);
     t.gemm_no_perm = std::getenv("FLUTE_GEMM_NO_PERM") != nullptr;
     t.gemm_ksplit = env_or("FLUTE_GEMM_KSPLIT", 0);
