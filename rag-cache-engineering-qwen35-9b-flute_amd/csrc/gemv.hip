@@ -446,6 +446,7 @@ flute_status launch_fast4(Plan &plan, hipStream_t stream) {
         if (per_cu > 0 && plan.p.split == 1 && (plan.p.nsegs == 1 || plan.p.silu_mul) &&
             plan.lds_bytes * per_cu <= (size_t)kLdsPerCU && gx > resident) {
             plan.p.slices = gx;
+            plan.p.xcd_runs = tuning().gemv_xcd && resident % 8 == 0;
             return launch_fast4_grid<LPGL, NW, PF, BF16, true>(plan, resident, stream);
         }
     }

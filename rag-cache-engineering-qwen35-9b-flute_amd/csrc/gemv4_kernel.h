@@ -297,7 +297,16 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     if constexpr (walk) {
         const int per = p.slices / (int)gridDim.x, extra = p.slices % (int)gridDim.x;
         const int b = (int)blockIdx.x;
-        if (per >= 4) {
+        if (per >= 4 && p.xcd_runs) {
+            // an eighth of the slices per XCD, divided evenly over its workgroups: the runs of an
+            // XCD lie side by side and every XCD streams the same share
+            const int x = b & 7, j = b >> 3, nx = (int)gridDim.x >> 3;
+            const int each = p.slices >> 3, odd = p.slices & 7;
+            const int first = x * each + min(x, odd), count = each + (x < odd ? 1 : 0);
+            const int per_x = count / nx, extra_x = count % nx;
+            sl = first + j * per_x + min(j, extra_x);
+            sl_end = sl + per_x + (j < extra_x ? 1 : 0);
+        } else if (per >= 4) {
             sl = b * per + min(b, extra);
             sl_end = sl + per + (b < extra ? 1 : 0);
         } else {
