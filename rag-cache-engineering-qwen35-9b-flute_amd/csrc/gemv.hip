@@ -496,7 +496,10 @@ flute_status launch_width(Plan &plan, hipStream_t stream) {
         }
     }
     const int nw = plan.threads / 64;
-    plan.p.xcd_runs = tuning().gemv_xcd && (plan.p.nsegs == 1 || plan.p.silu_mul) && plan.grid_x % 8 == 0;
+    // (a contiguous run of row slices per XCD: every weight's slices must come in eights)
+    plan.p.xcd_runs = tuning().gemv_xcd != 0;
+    for (int i = 0; i < plan.p.nsegs; ++i)
+        if (((plan.p.seg[i].N >> 7) * (256 >> plan.p.lpg_log2)) % 8 != 0) plan.p.xcd_runs = 0;
     // the lean kernel stages the activations once: gate and up must share input and rotation
     const bool one_input = !plan.p.silu_mul ||
                            (plan.p.seg[0].xsrc == plan.p.seg[1].xsrc &&

@@ -290,8 +290,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         // Consecutive workgroups go to consecutive XCDs.  Every XCD takes a contiguous run of slices
         // instead of every eighth one: the slices of a 128-row tile (their pieces of each 4 KB
         // index tile, their LUT row) then meet in one L2.  Measured 1 - 5 % (most on narrow outputs).
-        const int b = (int)blockIdx.x, per = (int)gridDim.x >> 3;
-        sl = (b & 7) * per + (b >> 3);
+        // (per weight of a grouped launch: the host checks that every weight's slices come in eights)
+        const int per = ((kp->seg[si0].N >> 7) * SPT) >> 3;
+        sl = (sl & 7) * per + (sl >> 3);
     }
     int sl_end = sl + 1, sl_step = 1;
     if constexpr (walk) {
