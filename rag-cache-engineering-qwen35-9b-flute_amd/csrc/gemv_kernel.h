@@ -925,8 +925,12 @@ __global__ void __launch_bounds__(kGemvMaxThreads, 3) gemv_kernel(const GemvPara
     gm.gpi = 64 >> p.lpg_log2;
     const int rw = lpg >> 1;                        // rows per workgroup
     const int spt = 128 / rw;                       // row slices per tile
-    const int sl = (int)blockIdx.x - sg.col0;
+    int sl = (int)blockIdx.x - sg.col0;
     const int spt_log2 = 8 - p.lpg_log2;            // spt = 128 / rw = 256 >> lpg_log2
+    if (p.xcd_runs) {                               // a contiguous run of this weight's slices per XCD
+        const int per = ((sg.N >> 7) << spt_log2) >> 3;
+        sl = (sl & 7) * per + (sl >> 3);
+    }
     gm.t = sl >> spt_log2;
     gm.cg0 = (sl & (spt - 1)) * (rw >> 3);
     gm.cg = gm.cg0 + (gm.l >> 4);
