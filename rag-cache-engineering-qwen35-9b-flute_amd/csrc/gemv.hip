@@ -767,3 +767,10 @@ int64_t flute_gemv_lds_bytes(const flute_linear *w, int split) {
 }
 
 }  // extern "C"
+
+#ifdef FLUTE_STAMPS
+// Instrumented builds only: where the lean kernel writes its phase times (NULL switches them off).
+extern "C" int flute_debug_gemv_stamps(void *buf) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_stamps), &buf, sizeof(buf));
+}
+#endif

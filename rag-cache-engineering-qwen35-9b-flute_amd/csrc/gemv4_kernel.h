@@ -52,6 +52,22 @@
 
 #include "gemv_kernel.h"
 
+#ifdef FLUTE_STAMPS
+// Instrumented builds only: per-wavefront phase times of the lean kernel (s_memrealtime, 10 ns
+// units), written to the buffer flute_debug_gemv_stamps() was given; gemv_phase_stamps.py reads them.
+// (One copy of the pointer per translation unit: the setter reaches the instantiations of gemv.hip.)
+__device__ long long *g_gemv_stamps = nullptr;
+#define FLUTE_GEMV_STAMP(slot)                                                                  \
+    do {                                                                                        \
+        if (g_gemv_stamps && (threadIdx.x & 63) == 0)                                           \
+            g_gemv_stamps[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x / 64) * 8 + \
+                          (threadIdx.x >> 6) * 8 + (slot)] =                                    \
+                (long long)__builtin_amdgcn_s_memrealtime();                                    \
+    } while (0)
+#else
+#define FLUTE_GEMV_STAMP(slot) do { } while (0)
+#endif
+
 namespace flute {
 
 typedef _Float16 gv_h8_t __attribute__((ext_vector_type(8)));
@@ -262,6 +278,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     constexpr int TAB1 = 16 * 256;
     constexpr int TAB_A = (TWO && BA == 1) ? TAB1 : (1 << (2 * BA)) * STRIDE;  // bytes of the first table
 
+    FLUTE_GEMV_STAMP(0);
     const GemvParams *kp = (const GemvParams *)(const void *)__builtin_amdgcn_kernarg_segment_ptr();
     warm_kernargs<(int)sizeof(GemvParams)>(kp);
     // several independent weights in one launch: the descriptor is picked by grid column
@@ -588,7 +605,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             q[n] = load_idx<BA>(qrow + (size_t)n * step + lane0);
             __builtin_amdgcn_sched_barrier(0);
         }
+        FLUTE_GEMV_STAMP(1);                        // (waits for the scalar loads: the LUT row is in)
         write_tables(lrow, lrowB, second0);
+        FLUTE_GEMV_STAMP(2);
         first_units(qrow, q, PF0);
         if (rot_inwave) {
             const int nst = 31 - __builtin_clz((unsigned)p.fht_block);
@@ -623,6 +642,7 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
             const int j = i < x_loads ? x_piece(i) : -1;
             if (j >= 0) stage8(j, xv[i]);
         }
+        FLUTE_GEMV_STAMP(3);
     } else if (x_plain) {
         // A long K range: two passes over this wavefront's pieces when a scale is needed
         // (the second one reads them from the cache).
@@ -972,8 +992,10 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         }
         // publishes the table; with the table kept, the alternating sum areas make it unnecessary
         if (!same_table) __syncthreads();
+        if (first) FLUTE_GEMV_STAMP(4);
 
         k_loop(q, qrow, lane0, step, slot, WA, q, qnext, lane0, step, WA, has_next);
+        if (!has_next) FLUTE_GEMV_STAMP(5);
 
         if (out_ends) end_of_output(so, par);
         if (!has_next) break;
@@ -996,7 +1018,9 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
         lut = lutn;
     }
     }
+    FLUTE_GEMV_STAMP(6);
     __syncthreads();
+    FLUTE_GEMV_STAMP(7);
 
     if (tid >= RW && p.split == 1) return;
     const bool owner = tid < RW;
