@@ -908,15 +908,22 @@ __global__ void __launch_bounds__(NW * 64, 3) gemv4_kernel(const GemvParams p) {
     //      a quad sum folds kt'; the activation scaling is undone here (exact). -----
     auto end_of_output = [&](int so_, int par_) {
         const bool keep = rb == kg;                 // here L >> 4 is the matrix row block
+        float v[8];
 #pragma unroll
         for (int a = 0; a < 8; ++a) {
             // lane kt' of a quad holds the wanted term in register kt': each register is
-            // read from its own lane of the quad, summed as (0 + 1) + (2 + 3)
-            const float v = (quad_lane<0x00>(acc[a][0]) + quad_lane<0x55>(acc[a][1])) +
-                            (quad_lane<0xAA>(acc[a][2]) + quad_lane<0xFF>(acc[a][3]));
-            if (keep && kt == 0)
-                red[par_ * (2 * NW * 32) + (so_ * NW + w) * 32 + rb * 8 + a] = ldexpf(v, xshift);
+            // read from its own lane of the quad, summed as (0 + 1) + (2 + 3).  The sums are
+            // formed by every lane, in front of the branch: there the lane reads fold into the
+            // additions (five instructions a sum instead of seven).
+            v[a] = (quad_lane<0x00>(acc[a][0]) + quad_lane<0x55>(acc[a][1])) +
+                   (quad_lane<0xAA>(acc[a][2]) + quad_lane<0xFF>(acc[a][3]));
+            asm volatile("" : "+v"(v[a]));
             acc[a] = (gv_f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        if (keep && kt == 0) {
+#pragma unroll
+            for (int a = 0; a < 8; ++a)
+                red[par_ * (2 * NW * 32) + (so_ * NW + w) * 32 + rb * 8 + a] = ldexpf(v[a], xshift);
         }
     };
     const auto WA = std::integral_constant<int, BA>();
