@@ -129,6 +129,11 @@ int plan_lds(GemmParams &p, const GemmShape &shape) {
         p.lean = shape.mb == 4 && ngrp == 1 && !tuning().gemm_no_lean;
         p.stage_off = lds_tables;
         lds_tables += shape.kw * shape.mw * (p.lean ? 8192 : 4096);
+        if (p.lean) {                            // one progress word per wavefront
+            p.prog_off = lds_tables;
+            lds_tables += 64;
+            p.balance = !tuning().gemm_no_balance;
+        }
     }
     const int slot_bytes = shape.mb * 8 * 64 * 16;
     const int lds_reduce = (shape.kw / 2) * shape.mw * slot_bytes;

@@ -35,12 +35,12 @@ int workspace_decision(size_t have_floats, size_t need_floats, size_t have_ints,
 // (flute_reload_tuning re-reads them): FLUTE_GEMV_RW, FLUTE_GEMV_WAVES,
 // FLUTE_GEMV_TABLE_LOG2, FLUTE_GEMV_PREROTATE, FLUTE_GEMV4_PF, FLUTE_GEMV_NO_FAST,
 // FLUTE_GEMV4_WALK, FLUTE_GEMV_XCD, FLUTE_GEMM_ROWS, FLUTE_GEMM_NO_PERM, FLUTE_GEMM_KSPLIT,
-// FLUTE_GEMM_NO_DIRECT, FLUTE_GEMM_NO_LEAN, FLUTE_FHT_STEPS.  Unset or empty = 0, except fht_steps and
+// FLUTE_GEMM_NO_DIRECT, FLUTE_GEMM_NO_LEAN, FLUTE_GEMM_NO_BALANCE, FLUTE_FHT_STEPS.  Unset or empty = 0, except fht_steps and
 // gemv4_walk = -1 (the launcher's own choice) and gemv_xcd = 1 (0: workgroup b of the lean GEMV takes
 // row slice b instead of a contiguous run of slices per XCD).
 struct Tuning {
     int gemv_rw, gemv_waves, gemv_table_log2, gemv_prerotate, gemv4_pf, gemv_no_fast, gemv4_walk, gemv_xcd;
-    int gemm_rows, gemm_no_perm, gemm_ksplit, gemm_no_direct, gemm_no_lean;
+    int gemm_rows, gemm_no_perm, gemm_ksplit, gemm_no_direct, gemm_no_lean, gemm_no_balance;
     int fht_steps;
 };
 const Tuning &tuning();
