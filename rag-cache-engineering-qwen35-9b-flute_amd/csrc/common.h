@@ -66,6 +66,15 @@ inline Segs make_segments(int K, int block) {
     return s;
 }
 
+// Activation image of the LUT GEMM, order of the 16-row blocks inside their groups of four: block
+// b of K tile g is stored at position b ^ image_block_xor(g, mode).  mode 0: as they come.  mode 1
+// (workgroups of four k ways): g & 3.  mode 2 (eight k ways): bit 2 and bit 1 of g swapped into
+// bits 1 and 0.  The k way that owns tile g then finds in position j the block its hand-overs at
+// the end of the kernel expect there (gemm_kernel.h).
+__host__ __device__ inline int image_block_xor(int g, int mode) {
+    return mode == 1 ? (g & 3) : mode == 2 ? (((g & 4) >> 1) | ((g & 2) >> 1)) : 0;
+}
+
 // A 64-bit address put together from two 32-bit halves that come out of builtins returning
 // `int` (__builtin_amdgcn_readfirstlane): each half is taken as unsigned first.  Converting the
 // int straight to uint64_t sign-extends it, and a low half with bit 31 set then sets all 32 upper

@@ -30,7 +30,7 @@ struct FhtParams {
     // GEMM's activation pre-pass would put it, Ap[g][j][m / 16][lane][8]; rows from M up
     // to the padded count are written as zeros.
     uint32_t *ap;
-    int ap_M, ap_mblk_pad, ap_bf16;
+    int ap_M, ap_mblk_pad, ap_bf16, ap_block_xor;
     int vec_io;     // x and out rows allow 16-byte accesses (16-bit types only)
     int vec_mul;    // signs and awq allow 16-byte loads
 };
@@ -54,7 +54,7 @@ __device__ __forceinline__ void store_operand_order(const FhtParams &p, int m, i
                                                     const uint16_t (&v)[8]) {
     const int g = k0 >> 6, kl = k0 & 63;
     const int jh = kl >> 5, s = ((kl >> 4) & 1) * 2 + ((kl >> 3) & 1);
-    const int64_t unit = ((int64_t)(g * 2 + jh) * p.ap_mblk_pad + (m >> 4)) * 64 + (m & 15);
+    const int64_t unit = ((int64_t)(g * 2 + jh) * p.ap_mblk_pad + ((m >> 4) ^ image_block_xor(g, p.ap_block_xor))) * 64 + (m & 15);
 #pragma unroll
     for (int kg = 0; kg < 4; ++kg)
         p.ap[(unit + kg * 16) * 4 + s] = (uint32_t)v[2 * kg] | ((uint32_t)v[2 * kg + 1] << 16);
@@ -412,6 +412,7 @@ flute_status fht_launch(const void *x, int64_t ldx, const float *signs, const fl
     p.ap = operand ? operand->ap : nullptr;
     p.ap_M = M;
     p.ap_mblk_pad = operand ? operand->mblk_pad : 0;
+    p.ap_block_xor = operand ? operand->block_xor : 0;
     p.ap_bf16 = operand ? operand->lut_bf16 : 0;
     const bool io16 = dtype != FLUTE_F32;
     p.vec_io = io16 && ((uintptr_t)x & 15) == 0 && ldx % 8 == 0 &&

@@ -140,6 +140,8 @@ int plan_lds(GemmParams &p, const GemmShape &shape) {
     const int lds_tile = shape.mw * shape.mb * 16 * 132 * 4 + 16;   // totals tile + ticket flag
     int lds = lds_tables > lds_reduce ? lds_tables : lds_reduce;
     if (lds_tile > lds) lds = lds_tile;
+    // the hand-overs between the k ways: eight 16 KB areas, then eight of 8 KB behind the totals tile
+    if (p.scatter && lds < 17 * 4096 + 8 * 8192) lds = 17 * 4096 + 8 * 8192;
     return lds;
 }
 
@@ -217,6 +219,13 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
     p.gper = (p.G + ksplit - 1) / ksplit;
     ksplit = (p.G + p.gper - 1) / p.gper;
     p.ksplit = ksplit;
+    // Four blocks per wavefront and K ranges that start on a multiple of the k ways: the image is
+    // written in the order the k ways want their blocks and they hand blocks to each other
+    // instead of reducing through a tree (gemm_kernel.h; FLUTE_GEMM_NO_HANDOVER keeps the tree).
+    p.scatter = 0;
+    if (shape.mb == 4 && shape.kw * shape.mw == 8 && p.gper % shape.kw == 0 && !tuning().gemm_no_handover)
+        p.scatter = shape.kw == 4 ? 1 : 2;
+    const int block_xor = p.scatter;
     FLUTE_REQUIRE(mchunks <= 65535 && ksplit <= 65535, FLUTE_ERR_UNSUPPORTED,
                   "flute_gemm: M=%d exceeds the grid", M);
 
@@ -271,7 +280,7 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
         }
     } else if (w->signs && w->R == 0 && !scale_rows) {
         // the rotation writes the operand image itself: one launch instead of two
-        FhtOperandOut image_out = {(uint32_t *)Ap, p.mblk_pad, (int)(w->lut_dtype == FLUTE_BF16)};
+        FhtOperandOut image_out = {(uint32_t *)Ap, p.mblk_pad, (int)(w->lut_dtype == FLUTE_BF16), block_xor};
         st = fht_launch(A, lda, w->signs, w->awq, nullptr, 0, M, w->K, act_dtype, 0, w->rot_block,
                         stream, &image_out);
         if (st != FLUTE_OK) return st;
@@ -299,12 +308,12 @@ extern "C" flute_status flute_gemm(const flute_linear *w, const void *A, void *C
                                (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
                                (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
                                rowshift, (const uint32_t *)w->lut1,
-                               (int)(((size_t)w->lut_rows << w->b1) * 2 / 64));
+                               (int)(((size_t)w->lut_rows << w->b1) * 2 / 64), block_xor);
         } else {
             hipLaunchKernelGGL(gemm_prep_kernel, dim3(blocks), dim3(256), 0, stream,
                                (const uint16_t *)A, Ap, M, lda, p.G, p.mblk_pad,
                                (int)(act_dtype == FLUTE_BF16), (int)(w->lut_dtype == FLUTE_BF16),
-                               (int)((((uintptr_t)A & 3) == 0) && (lda % 2 == 0)), rowshift);
+                               (int)((((uintptr_t)A & 3) == 0) && (lda % 2 == 0)), rowshift, block_xor);
         }
         FLUTE_HIP_CHECK(hipGetLastError());
     }

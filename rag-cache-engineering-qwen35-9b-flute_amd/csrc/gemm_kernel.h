@@ -70,6 +70,8 @@ struct GemmParams {
     int lean;              // 1: the launch uses the lean loop's instantiation
     int prog_off;          // lean loop: byte offset of one progress word per wavefront
     int balance;           // lean loop: 1 = the wavefront of a SIMD that is behind gets the higher priority
+    int scatter;           // four blocks per wavefront: the mode of image_block_xor the image was written with;
+                           // not 0: the k ways hand blocks to each other instead of reducing through the tree
     int nstreams;
     int M, N, K, G, gs, lut_rows, R;
     int mblk_total;        // ceil(M / 16)
@@ -86,18 +88,19 @@ struct GemmParams {
 };
 
 // Activation pre-pass: Ap[g][j][mb][lane][slot] in the LUT's 16-bit type.
+// block_xor: the mode of image_block_xor (common.h).
 __global__ void __launch_bounds__(256) gemm_prep_kernel(const uint16_t *A, u4_t *Ap, int M,
                                                         int64_t lda, int G, int mblk,
                                                         int in_bf16, int out_bf16, int pairs,
-                                                        const int *rowshift) {
+                                                        const int *rowshift, int block_xor) {
     const int64_t total = (int64_t)G * 2 * mblk * 64;
     for (int64_t o = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; o < total;
          o += (int64_t)gridDim.x * blockDim.x) {
         const int lane = (int)(o & 63);
         const int64_t rest = o >> 6;
-        const int mb = (int)(rest % mblk);
         const int gj = (int)(rest / mblk);
         const int g = gj >> 1, j = gj & 1;
+        const int mb = (int)(rest % mblk) ^ image_block_xor(g, block_xor);
         const int m = mb * 16 + (lane & 15), kg = lane >> 4;
         uint32_t out[4] = {0u, 0u, 0u, 0u};
         if (m < M) {
@@ -140,7 +143,8 @@ __global__ void __launch_bounds__(256) gemm_prep_quad_kernel(const uint16_t *A, 
                                                              int64_t lda, int G, int mblk,
                                                              int in_bf16, int out_bf16,
                                                              const int *rowshift,
-                                                             const uint32_t *warm, int warm_lines) {
+                                                             const uint32_t *warm, int warm_lines,
+                                                             int block_xor) {
     // The launch that follows starts with a chain of dependent loads (its arguments, then the
     // LUT rows): one thread per 64-byte line touches the LUT here, so that the rows come from
     // the memory-side cache there instead of from memory.
@@ -185,7 +189,7 @@ __global__ void __launch_bounds__(256) gemm_prep_quad_kernel(const uint16_t *A, 
         }
         FLUTE_TAKE(0) FLUTE_TAKE(1) FLUTE_TAKE(2) FLUTE_TAKE(3)
 #undef FLUTE_TAKE
-        Ap[((int64_t)gj * mblk + (m >> 4)) * 64 + q * 16 + (m & 15)] = out;
+        Ap[((int64_t)gj * mblk + ((m >> 4) ^ image_block_xor(gj >> 1, block_xor))) * 64 + q * 16 + (m & 15)] = out;
     }
 }
 
@@ -871,8 +875,58 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     FLUTE_STAMP(2);
     __syncthreads();                                    // tables are dead from here
     FLUTE_STAMP(3);
+    // Four blocks of rows per wavefront and the image in the order of image_block_xor: accumulator j
+    // of k way kw holds block j ^ x(kw).  Instead of the tree every wavefront hands the blocks it
+    // does not keep to the k way that keeps them: accumulators 2 and 3 to the k way whose 0 and 1
+    // they are, then accumulator 1 to the one whose 0 it is; with eight k ways two of them then
+    // hold the same block and the odd one gives its sums to the even one.  The same bytes cross
+    // LDS as in the tree and the sums are the same (every addition commutes), but all eight
+    // wavefronts move them, barriers go, and four or eight wavefronts write the totals tile.
+    const bool scattered = MB == 4 && KW * MW == 8 && p.scatter != 0;
+    if constexpr (MB == 4 && KW * MW == 8) {
+        if (scattered) {
+            constexpr int P1 = KW == 4 ? 2 : 4, P2 = KW == 4 ? 1 : 2;   // partners of the two hand-overs
+            f4_t *mine1 = red + (size_t)wave * 1024;
+            const f4_t *theirs1 = red + (size_t)(wave ^ P1) * 1024;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                mine1[i * 64 + lane] = acc[2][i];
+                mine1[(8 + i) * 64 + lane] = acc[3][i];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                acc[0][i] += theirs1[i * 64 + lane];
+                acc[1][i] += theirs1[(8 + i) * 64 + lane];
+            }
+            __syncthreads();
+            // second hand-over: behind the region the totals tile takes (17 * 4 KB from the start)
+            f4_t *mine2 = red + 4352 + (size_t)wave * 512;
+            const f4_t *theirs2 = red + 4352 + (size_t)(wave ^ P2) * 512;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) mine2[i * 64 + lane] = acc[1][i];
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[0][i] += theirs2[i * 64 + lane];
+            if constexpr (KW == 8) {
+                // k ways kw and kw ^ 1 hold the same block: between the (smaller) totals tile
+                // and the second hand-over's areas
+                f4_t *pair3 = red + 2176 + (size_t)(wave >> 1) * 512;
+                if (kw & 1) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) pair3[i * 64 + lane] = acc[0][i];
+                }
+                __syncthreads();
+                if (!(kw & 1)) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[0][i] += pair3[i * 64 + lane];
+                }
+            }
+        }
+    }
 #pragma unroll
     for (int step = KW / 2; step >= 1; step >>= 1) {
+        if (scattered) break;
         if (kw >= step && kw < 2 * step) {
             f4_t *slot = red + (size_t)((kw - step) * MW + mw) * (MB * 8 * 64);
 #pragma unroll
@@ -896,7 +950,16 @@ __global__ void __launch_bounds__(64 * KW * MW) gemm_kernel(const GemmParams p) 
     constexpr int ROWS = MW * MB * 16;                  // rows of C this workgroup owns
     constexpr int LDT = 128 + 4;                        // padded row: conflict-free both ways
     float *tile = (float *)smem;
-    if (kw == 0) {
+    if (scattered) {                                    // the totals of block x(kw) are in accumulator 0
+        if (KW == 4 || !(kw & 1)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = (mw * MB + image_block_xor(kw, p.scatter)) * 16 + rho;
+            const int n0 = (kg >> 1) * 64 + (i >> 1) * 16 + (i & 1) * 8 + (kg & 1) * 4;
+            *(f4_t *)(tile + row * LDT + n0) = acc[0][i];
+        }
+        }
+    } else if (kw == 0) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll

@@ -35,12 +35,13 @@ int workspace_decision(size_t have_floats, size_t need_floats, size_t have_ints,
 // (flute_reload_tuning re-reads them): FLUTE_GEMV_RW, FLUTE_GEMV_WAVES,
 // FLUTE_GEMV_TABLE_LOG2, FLUTE_GEMV_PREROTATE, FLUTE_GEMV4_PF, FLUTE_GEMV_NO_FAST,
 // FLUTE_GEMV4_WALK, FLUTE_GEMV_XCD, FLUTE_GEMM_ROWS, FLUTE_GEMM_NO_PERM, FLUTE_GEMM_KSPLIT,
-// FLUTE_GEMM_NO_DIRECT, FLUTE_GEMM_NO_LEAN, FLUTE_GEMM_NO_BALANCE, FLUTE_FHT_STEPS.  Unset or empty = 0, except fht_steps and
+// FLUTE_GEMM_NO_DIRECT, FLUTE_GEMM_NO_LEAN, FLUTE_GEMM_NO_BALANCE, FLUTE_GEMM_NO_HANDOVER,
+// FLUTE_FHT_STEPS.  Unset or empty = 0, except fht_steps and
 // gemv4_walk = -1 (the launcher's own choice) and gemv_xcd = 1 (0: workgroup b of the lean GEMV takes
 // row slice b instead of a contiguous run of slices per XCD).
 struct Tuning {
     int gemv_rw, gemv_waves, gemv_table_log2, gemv_prerotate, gemv4_pf, gemv_no_fast, gemv4_walk, gemv_xcd;
-    int gemm_rows, gemm_no_perm, gemm_ksplit, gemm_no_direct, gemm_no_lean, gemm_no_balance;
+    int gemm_rows, gemm_no_perm, gemm_ksplit, gemm_no_direct, gemm_no_lean, gemm_no_balance, gemm_no_handover;
     int fht_steps;
 };
 const Tuning &tuning();
@@ -52,6 +53,7 @@ struct FhtOperandOut {
     uint32_t *ap;       // Ap[g][j][m / 16][lane][4 dwords]
     int mblk_pad;       // 16-row blocks the image holds per half tile
     int lut_bf16;       // 16-bit type of the image
+    int block_xor;      // the mode of image_block_xor (common.h) the image is written with
 };
 flute_status fht_launch(const void *x, int64_t ldx, const float *signs, const float *awq, void *out,
                         int64_t ldo, int M, int K, int dtype, int adjoint, int block,

@@ -248,6 +248,7 @@ static void read_tuning() {
     t.gemm_no_direct = std::getenv("FLUTE_GEMM_NO_DIRECT") != nullptr;
     t.gemm_no_lean = std::getenv("FLUTE_GEMM_NO_LEAN") != nullptr;
     t.gemm_no_balance = std::getenv("FLUTE_GEMM_NO_BALANCE") != nullptr;
+    t.gemm_no_handover = std::getenv("FLUTE_GEMM_NO_HANDOVER") != nullptr;
     t.fht_steps = env_or("FLUTE_FHT_STEPS", -1);
     g_tuning = t;
 }

@@ -228,6 +228,47 @@ def test_lean_loop_is_bit_identical_to_the_scheduled_loop(tuning_env, N, K, M, l
     assert rel_l2(lean[7:8], y1) <= 4e-3                               # (bf16 outputs: one rounding each)
 
 
+@pytest.mark.parametrize("N,K,M,rot", [(12288, 4096, 256, False), (4096, 12288, 256, False), (4096, 12288, 200, True),
+                                       (12288, 4096, 1000, True), (1024, 4096, 300, True)])
+def test_hand_overs_between_the_k_ways_equal_the_tree(tuning_env, N, K, M, rot):
+    """Workgroups of four-block wavefronts end with hand-overs between their k ways (the activation
+    image is written with the blocks in the order those expect) and, under FLUTE_GEMM_NO_HANDOVER=1,
+    with the reduction tree over the image in plain order: the same additions, so equal bit for
+    bit, whether the image comes from the pre-pass or from the rotation that writes it itself,
+    with ragged M, four k ways (K = 4096) and eight (K = 12288)."""
+    import ctypes
+    from flute_extended import _lib
+    import fht
+    gen = torch.Generator(device=DEV).manual_seed(N + K + M)
+    blob = torch.randint(0, 256, (N * K // 2,), dtype=torch.uint8, device=DEV, generator=gen)
+    lut = (torch.randn(N // 128, 16, device=DEV, generator=gen) * 0.02).sort(dim=1).values.bfloat16().contiguous()
+    x = torch.randn(M, K, device=DEV, generator=gen).bfloat16()
+    signs = O.rotation_signs(K, 3).to(DEV) if rot else None
+    if N == 1024:
+        tuning_env("FLUTE_GEMM_ROWS", "128")
+    d = _lib.FluteLinear()
+    d.q1, d.lut1, d.q1_bytes = blob.data_ptr(), lut.data_ptr(), blob.numel()
+    d.N, d.K, d.b1, d.group_size, d.lut_rows, d.lut_dtype = N, K, 4, 128, N // 128, _lib.BF16
+    if rot:
+        d.signs = signs.data_ptr()
+
+    def run():
+        C = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+        st = _lib.lib.flute_gemm(ctypes.byref(d), x.data_ptr(), C.data_ptr(), M, K, N, _lib.BF16,
+                                 torch.cuda.current_stream().cuda_stream)
+        assert st == 0, _lib.last_error()
+        return C
+
+    handed = run()
+    tuning_env("FLUTE_GEMM_NO_HANDOVER", "1")
+    tree = run()
+    tuning_env("FLUTE_GEMM_NO_HANDOVER", None)
+    assert torch.equal(handed, tree)
+    xr = fht.fht_apply(x, signs, backend="kernel") if rot else x
+    y1 = fx.qgemm_gemv_splitk_stream(xr[M - 1:M], blob, lut, 4, 128)   # and against the M = 1 kernel
+    assert rel_l2(handed[M - 1:M], y1) <= 4e-3
+
+
 @pytest.mark.parametrize("kind", ["outliers", "tiny", "huge", "mixed"])
 @pytest.mark.parametrize("M,rows", [(8, None), (40, None), (130, "64"), (300, "128")])
 def test_gemm_bf16_activations_beyond_the_float16_range(tuning_env, kind, M, rows):
