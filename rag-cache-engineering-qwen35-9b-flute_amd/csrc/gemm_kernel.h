@@ -162,8 +162,15 @@ __global__ void __launch_bounds__(256) gemm_prep_quad_kernel(const uint16_t *A, 
          o += (int64_t)gridDim.x * blockDim.x) {
         const int q = (int)(o & 3);
         const int64_t wv = o >> 6;
-        const int gj = (int)(wv % segs);
-        const int m = (int)(wv / segs) * 16 + (int)((o >> 2) & 15);
+        int gj, mblock;
+        if (total >> 6 <= 0x7fffffff) {                 // uniform; a 64-bit division costs some hundred instructions
+            gj = (int)((uint32_t)wv % (uint32_t)segs);
+            mblock = (int)((uint32_t)wv / (uint32_t)segs);
+        } else {
+            gj = (int)(wv % segs);
+            mblock = (int)(wv / segs);
+        }
+        const int m = mblock * 16 + (int)((o >> 2) & 15);
         u4_t raw = {0u, 0u, 0u, 0u};
         if (m < M) {
             raw = *(const u4_t *)(A + (int64_t)m * lda + gj * 32 + q * 8);
